@@ -1,0 +1,190 @@
+/*
+ * torchrec_amd — C ABI of the MI355X (gfx950) quantized embedding inference
+ * kernels.  Plain C: raw device pointers, sizes and a hipStream_t (passed as
+ * void*).  The caller owns every buffer; calls are asynchronous on the given
+ * stream and re-entrant; nothing here synchronizes unless stated.
+ *
+ * Every entry point returns TRA_OK (0) or a negative TRA_ERR_* code and never
+ * throws.  tra_last_error() returns a thread-local message for the last
+ * failure.
+ *
+ * What each entry point replaces in the reference (pytorch/torchrec) is cited
+ * next to it; the operators themselves live in the un-vendored fbgemm_gpu
+ * dependency, so the citations are the reference's call sites.
+ */
+#ifndef TORCHREC_AMD_H_
+#define TORCHREC_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRA_OK 0
+#define TRA_ERR_INVALID_ARGUMENT (-1) /* bad dtype / shape / alignment / null */
+#define TRA_ERR_UNSUPPORTED (-2)      /* valid but not implemented            */
+#define TRA_ERR_HIP (-3)              /* a HIP runtime call failed            */
+#define TRA_ERR_NO_DEVICE (-4)        /* no gfx950 device / wrong arch        */
+#define TRA_ERR_TOO_LARGE (-5)        /* exceeds a documented limit           */
+
+/* Weight / output element types: values of fbgemm_gpu SparseType.as_int(). */
+#define TRA_FP32 0
+#define TRA_FP16 1
+#define TRA_INT8 2
+#define TRA_INT4 3
+#define TRA_INT2 4
+
+/* Pooling modes: values of fbgemm_gpu PoolingMode. */
+#define TRA_POOL_SUM 0
+#define TRA_POOL_MEAN 1
+#define TRA_POOL_NONE 2
+
+/* One table of a table-batched embedding (TBE) group.  Rows are packed in one
+ * uint8 buffer; table t starts at byte `offset`; row r starts at
+ * offset + r * row_bytes.  INT8/INT4/INT2 rows are
+ *   [fp16 scale][fp16 bias][payload dim*bits/8 bytes][pad]
+ * FP16/FP32 rows are [payload][pad].  row_bytes and offset must be multiples
+ * of 4.  (Reference: embedding_specs + row_alignment handed to
+ * IntNBitTableBatchedEmbeddingBagsCodegen, torchrec/quant/embedding_modules.py:
+ * 393-435.) */
+typedef struct tra_table_spec {
+  int64_t offset;
+  int64_t rows;
+  int32_t dim;
+  int32_t dtype;
+  int32_t row_bytes;
+  int32_t reserved;
+} tra_table_spec;
+
+typedef struct tra_tbe* tra_tbe_t;
+
+/* Library / device ------------------------------------------------------- */
+int tra_version(void);
+const char* tra_last_error(void);
+/* Name of the current device's architecture ("gfx950..."); TRA_ERR_NO_DEVICE
+ * if there is no usable GPU. */
+int tra_device_arch(char* buf, int buf_len);
+
+/* TBE group plan ---------------------------------------------------------- */
+/* Builds the immutable launch plan of one TBE group on the current device:
+ * per-feature descriptors (feature f reads table feature_table_map[f] and
+ * writes output columns D_offsets[f] .. D_offsets[f+1]) grouped by kernel
+ * class.  feature_positions (may be NULL = identity) gives, for each feature,
+ * the index of its bags in the offsets array passed to tra_tbe_forward: bag
+ * (f, b) is offsets[feature_positions[f] * B + b].  This is how a caller looks
+ * up from a KeyedJaggedTensor whose keys are ordered differently (or are a
+ * superset) without permuting it first; the reference permutes
+ * (torchrec/quant/embedding_modules.py:127-135, 535-537).  Allocates a few KB
+ * of device memory, released by tra_tbe_destroy.  Replaces the constructor of
+ * IntNBitTableBatchedEmbeddingBagsCodegen
+ * (torchrec/quant/embedding_modules.py:427-435, 828-836). */
+int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
+                   const int32_t* feature_table_map,
+                   const int32_t* feature_positions, int32_t num_features,
+                   tra_tbe_t* out);
+int tra_tbe_destroy(tra_tbe_t tbe);
+
+/* Pooled / sequence lookup.  Replaces
+ * IntNBitTableBatchedEmbeddingBagsCodegen.forward(indices, offsets,
+ * per_sample_weights) (torchrec/quant/embedding_modules.py:547-557 pooled,
+ * :938-942 sequence).
+ *   weights      device, the packed table buffer
+ *   indices      device [L], int32 or int64 (idx_is_i64); -1 = pruned id, skipped
+ *   offsets      device [K*B + 1] (K = number of input keys, F when
+ *                feature_positions is identity), same integer type; bag (f,b)
+ *                is offsets[p*B+b] .. offsets[p*B+b+1], p = feature_positions[f]
+ *   per_sample_weights device [L] fp32 or NULL (ignored for TRA_POOL_NONE)
+ *   out          device; pooled: [B, out_stride] elements, feature f at column
+ *                D_offsets[f]; TRA_POOL_NONE: [L, dim] (all features share dim)
+ *   out_dtype    TRA_FP32 or TRA_FP16
+ *   num_indices  L (sizes the TRA_POOL_NONE launch; pass -1 if unknown)
+ * Arithmetic per output column, ids in order: acc = fmaf(w*scale, q, acc +
+ * w*bias) (fp16/fp32 rows: acc = fmaf(w, x, acc)); MEAN multiplies by 1.0f/len;
+ * output rounded to nearest even.  Ids outside [0, rows) other than -1 are
+ * skipped and counted (tra_tbe_error_count). */
+int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
+                    const void* offsets, int32_t idx_is_i64,
+                    const float* per_sample_weights, int32_t batch_size,
+                    int64_t num_indices, int32_t pooling_mode,
+                    int32_t out_dtype, void* out, int64_t out_stride,
+                    void* stream);
+
+/* Number of out-of-range ids seen by forwards on this plan since the last
+ * call (synchronizes the stream; resets the counter).  Stands in for
+ * fbgemm_gpu's bounds_check_indices. */
+int tra_tbe_error_count(tra_tbe_t tbe, void* stream, int64_t* count);
+
+/* Index math -------------------------------------------------------------- */
+/* offsets[0] = 0, offsets[i+1] = sum(lengths[0..i]).  n <= 2^31-1 elements.
+ * Replaces torch.ops.fbgemm.asynchronous_complete_cumsum
+ * (torchrec/sparse/jagged_tensor.py:79-80).  workspace: device scratch of
+ * tra_cumsum_workspace_bytes(n) bytes (may be NULL when that is 0). */
+int64_t tra_cumsum_workspace_bytes(int64_t n);
+int tra_cumsum(const void* lengths, int64_t n, int32_t is_i64, void* offsets,
+               void* workspace, void* stream);
+
+/* Per-feature totals: out[f] = sum(lengths[f*B .. (f+1)*B)) as int64.
+ * Replaces torch.sum(lengths.view(F, B), 1) in KJT.length_per_key
+ * (torchrec/sparse/jagged_tensor.py:1201-1212). */
+int tra_length_per_key(const void* lengths, int32_t num_features,
+                       int32_t batch_size, int32_t is_i64, int64_t* out,
+                       void* stream);
+
+/* Feature permutation of a KJT.  lengths is [T, B]; out_lengths[t', :] =
+ * lengths[permute[t'], :]; values (and weights) segments follow in the new
+ * order.  in_offsets / out_offsets are the complete cumsums ([T*B+1] /
+ * [T'*B+1], same integer type as lengths) of lengths / out_lengths, computed by
+ * the caller with tra_cumsum.  value_bytes is 4 or 8.  Replaces
+ * torch.ops.fbgemm.permute_2D_sparse_data
+ * (torchrec/sparse/jagged_tensor.py:2573-2583). */
+int tra_permute_2d_lengths(const int32_t* permute, int32_t num_out_features,
+                           int32_t num_features, int32_t batch_size,
+                           const void* lengths, int32_t is_i64,
+                           void* out_lengths, void* stream);
+int tra_permute_2d_data(const int32_t* permute, int32_t num_out_features,
+                        int32_t batch_size, const void* in_offsets,
+                        const void* out_offsets, int32_t is_i64,
+                        const void* values, int32_t value_bytes,
+                        const float* weights, void* out_values,
+                        float* out_weights, void* stream);
+
+/* Block bucketization of ids (row-wise sharding index math).  Replaces
+ * torch.ops.fbgemm.block_bucketize_sparse_features
+ * (torchrec/distributed/embedding_sharding.py:153-198).
+ * Step 1 writes new_lengths [W*F*B] (bucket-major); the caller cumsums them
+ * into new_offsets [W*F*B+1]; step 2 scatters ids (id % block_size, or the id
+ * itself if keep_orig_idx), weights, and optionally unbucketize_permute [L]
+ * (output position of each input id, -1 if dropped).  Order inside one
+ * (bucket, f, b) is the input order.  offsets is the complete cumsum of
+ * lengths; cursor_workspace is device scratch of W*F*B int64. */
+int tra_bucketize_lengths(const void* offsets, const void* indices,
+                          int32_t is_i64, const int64_t* block_sizes,
+                          int32_t num_features, int32_t batch_size,
+                          int32_t num_buckets, void* new_lengths, void* stream);
+int tra_bucketize_scatter(const void* offsets, const void* indices,
+                          int32_t is_i64, const float* weights,
+                          const int64_t* block_sizes, int32_t num_features,
+                          int32_t batch_size, int32_t num_buckets,
+                          int32_t keep_orig_idx, const void* new_offsets,
+                          int64_t* cursor_workspace, void* new_indices,
+                          float* new_weights, int64_t* unbucketize_permute,
+                          void* stream);
+
+/* Row-wise quantization --------------------------------------------------- */
+/* fp32 [rows, dim] -> packed TBE rows (header-first, row_bytes stride) written
+ * straight into the table buffer at `out`; bits in {8, 4, 2}.  Same bytes as
+ * torch.ops.fbgemm.FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf followed by
+ * the reference's trailer split (torchrec/quant/embedding_modules.py:261-276),
+ * with scale/bias moved to the row header. */
+int tra_quantize_rows(const float* in, int64_t rows, int32_t dim, int32_t bits,
+                      uint8_t* out, int32_t row_bytes, void* stream);
+/* Same input, fbgemm's own output format: [rows, dim*bits/8 + 4] with the
+ * fp16 scale/bias at the END of each row. */
+int tra_quantize_rows_sbhalf(const float* in, int64_t rows, int32_t dim,
+                             int32_t bits, uint8_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCHREC_AMD_H_ */

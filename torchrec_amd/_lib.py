@@ -1,0 +1,115 @@
+"""ctypes binding of ``libtorchrec_amd.so`` (the C ABI in include/torchrec_amd.h).
+
+The library is built in-tree by ``torchrec_amd/csrc/Makefile`` (``build()`` in
+``__graft_entry__.py`` or ``python -m torchrec_amd.build``).  There is no other
+implementation behind these calls: if the library is missing, or there is no
+gfx950 device, every entry point here raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtorchrec_amd.so")
+
+# Names every build must export (checked by tests/test_capi_symbols.py).
+EXPORTED_SYMBOLS = [
+    "tra_version",
+    "tra_last_error",
+    "tra_device_arch",
+    "tra_tbe_create",
+    "tra_tbe_destroy",
+    "tra_tbe_forward",
+    "tra_tbe_error_count",
+    "tra_cumsum_workspace_bytes",
+    "tra_cumsum",
+    "tra_length_per_key",
+    "tra_permute_2d_lengths",
+    "tra_permute_2d_data",
+    "tra_bucketize_lengths",
+    "tra_bucketize_scatter",
+    "tra_quantize_rows",
+    "tra_quantize_rows_sbhalf",
+]
+
+TRA_OK = 0
+FP32, FP16, INT8, INT4, INT2 = 0, 1, 2, 3, 4
+POOL_SUM, POOL_MEAN, POOL_NONE = 0, 1, 2
+
+
+class TableSpec(ctypes.Structure):
+    _fields_ = [
+        ("offset", ctypes.c_int64),
+        ("rows", ctypes.c_int64),
+        ("dim", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("row_bytes", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class TorchrecAmdError(RuntimeError):
+    pass
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded kernel library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TorchrecAmdError(
+                f"{LIB_PATH} is missing: build it with `make -C torchrec_amd/csrc` "
+                "(hipcc, --offload-arch=gfx950). torchrec_amd has no other backend."
+            )
+        l = ctypes.CDLL(LIB_PATH)
+        vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+        l.tra_version.restype = ctypes.c_int
+        l.tra_last_error.restype = ctypes.c_char_p
+        l.tra_device_arch.argtypes = [ctypes.c_char_p, ctypes.c_int]
+        l.tra_tbe_create.argtypes = [ctypes.POINTER(TableSpec), i32, ctypes.POINTER(i32), ctypes.POINTER(i32), i32, ctypes.POINTER(vp)]
+        l.tra_tbe_destroy.argtypes = [vp]
+        l.tra_tbe_forward.argtypes = [vp, vp, vp, vp, i32, vp, i32, i64, i32, i32, vp, i64, vp]
+        l.tra_tbe_error_count.argtypes = [vp, vp, ctypes.POINTER(i64)]
+        l.tra_cumsum_workspace_bytes.argtypes = [i64]
+        l.tra_cumsum_workspace_bytes.restype = i64
+        l.tra_cumsum.argtypes = [vp, i64, i32, vp, vp, vp]
+        l.tra_length_per_key.argtypes = [vp, i32, i32, i32, vp, vp]
+        l.tra_permute_2d_lengths.argtypes = [vp, i32, i32, i32, vp, i32, vp, vp]
+        l.tra_permute_2d_data.argtypes = [vp, i32, i32, vp, vp, i32, vp, i32, vp, vp, vp, vp]
+        l.tra_bucketize_lengths.argtypes = [vp, vp, i32, vp, i32, i32, i32, vp, vp]
+        l.tra_bucketize_scatter.argtypes = [vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp]
+        l.tra_quantize_rows.argtypes = [vp, i64, i32, i32, vp, i32, vp]
+        l.tra_quantize_rows_sbhalf.argtypes = [vp, i64, i32, i32, vp, vp]
+        _lib = l
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != TRA_OK:
+        msg = lib().tra_last_error().decode("utf-8", "replace")
+        raise TorchrecAmdError(f"torchrec_amd error {rc}: {msg}")
+
+
+def require_gpu(t: torch.Tensor, what: str) -> None:
+    """The kernels run on MI355X only; there is no host implementation."""
+    if t.device.type != "cuda":
+        raise TorchrecAmdError(
+            f"{what}: tensor is on {t.device}; torchrec_amd runs this on a gfx950 GPU only"
+        )
+
+
+def ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    if t is None:
+        return ctypes.c_void_p(0)
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def current_stream(device: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)

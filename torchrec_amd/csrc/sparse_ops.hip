@@ -1,0 +1,462 @@
+// Index math around the lookup (offsets, per-key totals, feature permutation,
+// block bucketization) and the row-wise quantizer.  Integer results are
+// bit-exact by construction; these are bandwidth-trivial next to the gather.
+#include <hip/hip_fp16.h>
+
+#include "tra_common.h"
+
+namespace tra {
+
+constexpr int kScanThreads = 256;
+constexpr int kScanItems = 16;
+constexpr int kScanTile = kScanThreads * kScanItems;
+
+template <typename T>
+__device__ __forceinline__ int64_t ld(const void* p, int64_t i) {
+  return (int64_t) reinterpret_cast<const T*>(p)[i];
+}
+template <typename T>
+__device__ __forceinline__ void st(void* p, int64_t i, int64_t v) {
+  reinterpret_cast<T*>(p)[i] = (T)v;
+}
+
+__device__ __forceinline__ int64_t wave_sum(int64_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Block-wide sum; result valid in every thread.  `smem` holds >= 4 int64.
+__device__ __forceinline__ int64_t block_sum(int64_t v, int64_t* smem) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWaveSize;
+  __syncthreads();
+  if ((threadIdx.x & (kWaveSize - 1)) == 0) smem[wave] = v;
+  __syncthreads();
+  int64_t t = 0;
+  for (int w = 0; w < (int)(blockDim.x / kWaveSize); ++w) t += smem[w];
+  return t;
+}
+
+// ---- complete cumsum --------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kScanThreads) void tile_sums_kernel(const void* in, int64_t n,
+                                                                  int64_t* sums) {
+  __shared__ int64_t smem[kScanThreads / kWaveSize];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile;
+  int64_t v = 0;
+  for (int i = threadIdx.x; i < kScanTile; i += kScanThreads)
+    if (base + i < n) v += ld<T>(in, base + i);
+  v = block_sum(v, smem);
+  if (threadIdx.x == 0) sums[blockIdx.x] = v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kScanThreads) void scan_tiles_kernel(const void* in, int64_t n,
+                                                                   const int64_t* sums, void* out) {
+  __shared__ int64_t smem[kScanThreads / kWaveSize];
+  __shared__ int64_t wave_tot[kScanThreads / kWaveSize];
+  // Sum of all earlier tiles.
+  int64_t prefix = 0;
+  if (sums) {
+    for (int i = threadIdx.x; i < (int)blockIdx.x; i += kScanThreads) prefix += sums[i];
+    prefix = block_sum(prefix, smem);
+  }
+  // Each thread owns kScanItems consecutive elements.
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  int64_t x[kScanItems];
+  int64_t tsum = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    x[i] = base + i < n ? ld<T>(in, base + i) : 0;
+    tsum += x[i];
+  }
+  // Exclusive scan of the per-thread sums: wave scan, then wave totals.
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  int64_t inc = tsum;
+#pragma unroll
+  for (int off = 1; off < kWaveSize; off <<= 1) {
+    const int64_t o = __shfl_up(inc, off, 64);
+    if (lane >= off) inc += o;
+  }
+  if (lane == kWaveSize - 1) wave_tot[wave] = inc;
+  __syncthreads();
+  int64_t wprefix = 0;
+  for (int w = 0; w < wave; ++w) wprefix += wave_tot[w];
+  int64_t run = prefix + wprefix + inc - tsum;
+  if (blockIdx.x == 0 && threadIdx.x == 0) st<T>(out, 0, 0);
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    run += x[i];
+    if (base + i < n) st<T>(out, base + i + 1, run);
+  }
+}
+
+// ---- per-key totals ---------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kScanThreads) void length_per_key_kernel(const void* lengths,
+                                                                       int32_t B, int64_t* out) {
+  __shared__ int64_t smem[kScanThreads / kWaveSize];
+  const int64_t base = (int64_t)blockIdx.x * B;
+  int64_t v = 0;
+  for (int i = threadIdx.x; i < B; i += kScanThreads) v += ld<T>(lengths, base + i);
+  v = block_sum(v, smem);
+  if (threadIdx.x == 0) out[blockIdx.x] = v;
+}
+
+// ---- feature permutation ----------------------------------------------------
+template <typename T>
+__global__ void permute_lengths_kernel(const int32_t* permute, int64_t total, int32_t B,
+                                       const void* lengths, void* out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t tp = i / B;
+  const int64_t b = i - tp * B;
+  st<T>(out, i, ld<T>(lengths, (int64_t)permute[tp] * B + b));
+}
+
+// All values of one feature are contiguous on both sides, so each output
+// feature is one straight copy.  grid = (blocks per feature, T').
+template <typename OffT, typename ValT>
+__global__ void permute_data_kernel(const int32_t* permute, int32_t B, const void* in_off,
+                                    const void* out_off, const ValT* values, const float* weights,
+                                    ValT* out_values, float* out_weights) {
+  const int tp = blockIdx.y;
+  const int64_t src = ld<OffT>(in_off, (int64_t)permute[tp] * B);
+  const int64_t dst = ld<OffT>(out_off, (int64_t)tp * B);
+  const int64_t n = ld<OffT>(out_off, (int64_t)(tp + 1) * B) - dst;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    out_values[dst + i] = values[src + i];
+    if (weights) out_weights[dst + i] = weights[src + i];
+  }
+}
+
+// ---- block bucketization ----------------------------------------------------
+// One thread per bag (f, b); a bag's ids are visited in order, so the order
+// inside one (bucket, f, b) is the input order.
+template <typename T>
+__global__ void bucketize_lengths_kernel(const void* offsets, const void* indices,
+                                         const int64_t* block_sizes, int32_t B, int64_t n,
+                                         int32_t W, void* new_lengths) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  T* nl = reinterpret_cast<T*>(new_lengths);
+  for (int p = 0; p < W; ++p) nl[(int64_t)p * n + i] = 0;
+  const int64_t bs = block_sizes[i / B];
+  const int64_t s = ld<T>(offsets, i), e = ld<T>(offsets, i + 1);
+  for (int64_t j = s; j < e; ++j) {
+    const int64_t id = ld<T>(indices, j);
+    const uint64_t p = (uint64_t)id / (uint64_t)bs;
+    if (p < (uint64_t)W) nl[(int64_t)p * n + i] += 1;
+  }
+}
+
+template <typename T>
+__global__ void bucketize_scatter_kernel(const void* offsets, const void* indices,
+                                         const float* weights, const int64_t* block_sizes,
+                                         int32_t B, int64_t n, int32_t W, int keep_orig,
+                                         const void* new_offsets, int64_t* cursor,
+                                         void* new_indices, float* new_weights,
+                                         int64_t* unbucketize_permute) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  for (int p = 0; p < W; ++p) cursor[(int64_t)p * n + i] = ld<T>(new_offsets, (int64_t)p * n + i);
+  const int64_t bs = block_sizes[i / B];
+  const int64_t s = ld<T>(offsets, i), e = ld<T>(offsets, i + 1);
+  for (int64_t j = s; j < e; ++j) {
+    const int64_t id = ld<T>(indices, j);
+    const uint64_t p = (uint64_t)id / (uint64_t)bs;
+    if (p >= (uint64_t)W) {
+      if (unbucketize_permute) unbucketize_permute[j] = -1;
+      continue;
+    }
+    const int64_t pos = cursor[(int64_t)p * n + i]++;
+    st<T>(new_indices, pos, keep_orig ? id : (int64_t)((uint64_t)id % (uint64_t)bs));
+    if (weights) new_weights[pos] = weights[j];
+    if (unbucketize_permute) unbucketize_permute[j] = pos;
+  }
+}
+
+// ---- row-wise N-bit quantization -------------------------------------------
+// One wave per row.  Same operation order as fbgemm's
+// FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf: min/max, bias = fp16(min),
+// scale = fp16((max - bias) / (2^bits - 1)), q = clamp(rint((x - bias) * (1/scale))).
+// header_first: TBE row [scale][bias][payload]; otherwise fbgemm's trailer row.
+template <int BITS>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const float* in, int64_t rows,
+                                                            int32_t dim, uint8_t* out,
+                                                            int64_t row_bytes, int header_first) {
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int64_t r = (int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
+  if (r >= rows) return;
+  const float* x = in + r * dim;
+  float mn = x[0], mx = x[0];
+  for (int c = lane; c < dim; c += kWaveSize) {
+    const float v = x[c];
+    mn = v < mn ? v : mn;
+    mx = v > mx ? v : mx;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float a = __shfl_xor(mn, off, 64), b = __shfl_xor(mx, off, 64);
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+  }
+  constexpr int kQMax = (1 << BITS) - 1;
+  constexpr int kEpb = 8 / BITS;
+  const __half bias_h = __float2half_rn(mn);
+  const float bias = __half2float(bias_h);
+  const float range = mx - bias;
+  float scale = range == 0.0f ? 1.0f : range / (float)kQMax;
+  scale = __half2float(__float2half_rn(scale));
+  if (scale == 0.0f) scale = 1.0f;
+  float inv = 1.0f / scale;
+  if (__builtin_isinf(inv)) {
+    scale = 1.0f;
+    inv = 1.0f;
+  }
+  const __half scale_h = __float2half_rn(scale);
+  const int payload = dim / kEpb;
+  uint8_t* o = out + r * row_bytes;
+  uint8_t* pay = header_first ? o + 4 : o;
+  uint8_t* hdr = header_first ? o : o + payload;
+  for (int byte = lane; byte < payload; byte += kWaveSize) {
+    uint32_t packed = 0;
+#pragma unroll
+    for (int e = 0; e < kEpb; ++e) {
+      const float t = (x[byte * kEpb + e] - bias) * inv;
+      float q = __builtin_rintf(t);
+      q = q < 0.0f ? 0.0f : q;
+      q = q > (float)kQMax ? (float)kQMax : q;
+      packed |= (uint32_t)(int)q << (e * BITS);
+    }
+    pay[byte] = (uint8_t)packed;
+  }
+  if (lane == 0) {
+    const uint16_t s = __half_as_ushort(scale_h), b = __half_as_ushort(bias_h);
+    hdr[0] = (uint8_t)(s & 0xff);
+    hdr[1] = (uint8_t)(s >> 8);
+    hdr[2] = (uint8_t)(b & 0xff);
+    hdr[3] = (uint8_t)(b >> 8);
+  }
+}
+
+static int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, what);
+  return TRA_OK;
+}
+
+static int quantize_impl(const float* in, int64_t rows, int32_t dim, int32_t bits, uint8_t* out,
+                         int64_t row_bytes, int header_first, hipStream_t s) {
+  if (bits != 8 && bits != 4 && bits != 2) {
+    set_error("quantize: bits must be 8, 4 or 2 (got %d)", bits);
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (dim <= 0 || dim % (8 / bits) != 0 || rows < 0 || row_bytes < dim * bits / 8 + 4) {
+    set_error("quantize: bad dim %d / row_bytes %lld for %d bits", dim, (long long)row_bytes, bits);
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (rows == 0) return TRA_OK;
+  if (!in || !out) {
+    set_error("quantize: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffff) {
+    set_error("quantize: too many rows in one call");
+    return TRA_ERR_TOO_LARGE;
+  }
+  dim3 g((unsigned)blocks), b(256);
+  if (bits == 8)
+    hipLaunchKernelGGL(quantize_rows_kernel<8>, g, b, 0, s, in, rows, dim, out, row_bytes, header_first);
+  else if (bits == 4)
+    hipLaunchKernelGGL(quantize_rows_kernel<4>, g, b, 0, s, in, rows, dim, out, row_bytes, header_first);
+  else
+    hipLaunchKernelGGL(quantize_rows_kernel<2>, g, b, 0, s, in, rows, dim, out, row_bytes, header_first);
+  return check_launch("quantize_rows");
+}
+
+}  // namespace tra
+
+using namespace tra;
+
+extern "C" {
+
+int64_t tra_cumsum_workspace_bytes(int64_t n) {
+  const int64_t tiles = (n + kScanTile - 1) / kScanTile;
+  return tiles > 1 ? tiles * (int64_t)sizeof(int64_t) : 0;
+}
+
+int tra_cumsum(const void* lengths, int64_t n, int32_t is_i64, void* offsets, void* workspace,
+               void* stream) {
+  if (n < 0 || !offsets || (n > 0 && !lengths)) {
+    set_error("tra_cumsum: bad argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (n > 0x7fffffffLL) {
+    set_error("tra_cumsum: n too large");
+    return TRA_ERR_TOO_LARGE;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t tiles = n == 0 ? 1 : (n + kScanTile - 1) / kScanTile;
+  int64_t* sums = nullptr;
+  if (tiles > 1) {
+    if (!workspace) {
+      set_error("tra_cumsum: workspace of %lld bytes required",
+                (long long)tra_cumsum_workspace_bytes(n));
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+    sums = (int64_t*)workspace;
+    if (is_i64)
+      hipLaunchKernelGGL(tile_sums_kernel<int64_t>, dim3((unsigned)tiles), dim3(kScanThreads), 0, s,
+                         lengths, n, sums);
+    else
+      hipLaunchKernelGGL(tile_sums_kernel<int32_t>, dim3((unsigned)tiles), dim3(kScanThreads), 0, s,
+                         lengths, n, sums);
+  }
+  if (is_i64)
+    hipLaunchKernelGGL(scan_tiles_kernel<int64_t>, dim3((unsigned)tiles), dim3(kScanThreads), 0, s,
+                       lengths, n, sums, offsets);
+  else
+    hipLaunchKernelGGL(scan_tiles_kernel<int32_t>, dim3((unsigned)tiles), dim3(kScanThreads), 0, s,
+                       lengths, n, sums, offsets);
+  return check_launch("tra_cumsum");
+}
+
+int tra_length_per_key(const void* lengths, int32_t num_features, int32_t batch_size,
+                       int32_t is_i64, int64_t* out, void* stream) {
+  if (num_features < 0 || batch_size < 0 || (num_features > 0 && (!out || (!lengths && batch_size)))) {
+    set_error("tra_length_per_key: bad argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (num_features == 0) return TRA_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_i64)
+    hipLaunchKernelGGL(length_per_key_kernel<int64_t>, dim3(num_features), dim3(kScanThreads), 0, s,
+                       lengths, batch_size, out);
+  else
+    hipLaunchKernelGGL(length_per_key_kernel<int32_t>, dim3(num_features), dim3(kScanThreads), 0, s,
+                       lengths, batch_size, out);
+  return check_launch("tra_length_per_key");
+}
+
+int tra_permute_2d_lengths(const int32_t* permute, int32_t num_out_features, int32_t num_features,
+                           int32_t batch_size, const void* lengths, int32_t is_i64,
+                           void* out_lengths, void* stream) {
+  (void)num_features;
+  const int64_t total = (int64_t)num_out_features * batch_size;
+  if (num_out_features < 0 || batch_size < 0) {
+    set_error("tra_permute_2d_lengths: bad argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (total == 0) return TRA_OK;
+  if (!permute || !lengths || !out_lengths) {
+    set_error("tra_permute_2d_lengths: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  dim3 g((unsigned)((total + 255) / 256)), b(256);
+  if (is_i64)
+    hipLaunchKernelGGL(permute_lengths_kernel<int64_t>, g, b, 0, s, permute, total, batch_size,
+                       lengths, out_lengths);
+  else
+    hipLaunchKernelGGL(permute_lengths_kernel<int32_t>, g, b, 0, s, permute, total, batch_size,
+                       lengths, out_lengths);
+  return check_launch("tra_permute_2d_lengths");
+}
+
+int tra_permute_2d_data(const int32_t* permute, int32_t num_out_features, int32_t batch_size,
+                        const void* in_offsets, const void* out_offsets, int32_t is_i64,
+                        const void* values, int32_t value_bytes, const float* weights,
+                        void* out_values, float* out_weights, void* stream) {
+  if (num_out_features < 0 || batch_size < 0 || (value_bytes != 4 && value_bytes != 8)) {
+    set_error("tra_permute_2d_data: bad argument (value_bytes must be 4 or 8)");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (num_out_features == 0 || batch_size == 0) return TRA_OK;
+  if (!permute || !in_offsets || !out_offsets || (weights && !out_weights)) {
+    set_error("tra_permute_2d_data: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  dim3 g(64, (unsigned)num_out_features), b(256);
+#define GO(OFF, VAL)                                                                          \
+  hipLaunchKernelGGL((permute_data_kernel<OFF, VAL>), g, b, 0, s, permute, batch_size,        \
+                     in_offsets, out_offsets, (const VAL*)values, weights, (VAL*)out_values,  \
+                     out_weights)
+  if (is_i64) {
+    if (value_bytes == 8) GO(int64_t, int64_t); else GO(int64_t, int32_t);
+  } else {
+    if (value_bytes == 8) GO(int32_t, int64_t); else GO(int32_t, int32_t);
+  }
+#undef GO
+  return check_launch("tra_permute_2d_data");
+}
+
+int tra_bucketize_lengths(const void* offsets, const void* indices, int32_t is_i64,
+                          const int64_t* block_sizes, int32_t num_features, int32_t batch_size,
+                          int32_t num_buckets, void* new_lengths, void* stream) {
+  const int64_t n = (int64_t)num_features * batch_size;
+  if (num_features < 0 || batch_size < 0 || num_buckets <= 0) {
+    set_error("tra_bucketize_lengths: bad argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (n == 0) return TRA_OK;
+  if (!offsets || !block_sizes || !new_lengths) {
+    set_error("tra_bucketize_lengths: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  dim3 g((unsigned)((n + 127) / 128)), b(128);
+  if (is_i64)
+    hipLaunchKernelGGL(bucketize_lengths_kernel<int64_t>, g, b, 0, s, offsets, indices, block_sizes,
+                       batch_size, n, num_buckets, new_lengths);
+  else
+    hipLaunchKernelGGL(bucketize_lengths_kernel<int32_t>, g, b, 0, s, offsets, indices, block_sizes,
+                       batch_size, n, num_buckets, new_lengths);
+  return check_launch("tra_bucketize_lengths");
+}
+
+int tra_bucketize_scatter(const void* offsets, const void* indices, int32_t is_i64,
+                          const float* weights, const int64_t* block_sizes, int32_t num_features,
+                          int32_t batch_size, int32_t num_buckets, int32_t keep_orig_idx,
+                          const void* new_offsets, int64_t* cursor_workspace, void* new_indices,
+                          float* new_weights, int64_t* unbucketize_permute, void* stream) {
+  const int64_t n = (int64_t)num_features * batch_size;
+  if (num_features < 0 || batch_size < 0 || num_buckets <= 0) {
+    set_error("tra_bucketize_scatter: bad argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (n == 0) return TRA_OK;
+  if (!offsets || !block_sizes || !new_offsets || !cursor_workspace || (weights && !new_weights)) {
+    set_error("tra_bucketize_scatter: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  dim3 g((unsigned)((n + 127) / 128)), b(128);
+  if (is_i64)
+    hipLaunchKernelGGL(bucketize_scatter_kernel<int64_t>, g, b, 0, s, offsets, indices, weights,
+                       block_sizes, batch_size, n, num_buckets, keep_orig_idx, new_offsets,
+                       cursor_workspace, new_indices, new_weights, unbucketize_permute);
+  else
+    hipLaunchKernelGGL(bucketize_scatter_kernel<int32_t>, g, b, 0, s, offsets, indices, weights,
+                       block_sizes, batch_size, n, num_buckets, keep_orig_idx, new_offsets,
+                       cursor_workspace, new_indices, new_weights, unbucketize_permute);
+  return check_launch("tra_bucketize_scatter");
+}
+
+int tra_quantize_rows(const float* in, int64_t rows, int32_t dim, int32_t bits, uint8_t* out,
+                      int32_t row_bytes, void* stream) {
+  return quantize_impl(in, rows, dim, bits, out, row_bytes, 1, (hipStream_t)stream);
+}
+
+int tra_quantize_rows_sbhalf(const float* in, int64_t rows, int32_t dim, int32_t bits,
+                             uint8_t* out, void* stream) {
+  const int64_t rb = bits > 0 && bits <= 8 ? (int64_t)dim * bits / 8 + 4 : 0;
+  return quantize_impl(in, rows, dim, bits, out, rb, 0, (hipStream_t)stream);
+}
+
+}  // extern "C"

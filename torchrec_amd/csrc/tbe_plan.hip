@@ -1,0 +1,327 @@
+// Host side of the TBE lookup: plan construction (tra_tbe_create) and launch
+// (tra_tbe_forward), plus the small library-level entry points.
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <string>
+
+#include "tbe_lookup_impl.h"
+
+namespace tra {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  set_error("%s: %s", what, hipGetErrorString(e));
+  return TRA_ERR_HIP;
+}
+
+// Explicit specializations live in tbe_lookup_<dtype>.hip.
+template <>
+int launch_lookup<TRA_INT8>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+template <>
+int launch_lookup<TRA_INT4>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+template <>
+int launch_lookup<TRA_INT2>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+template <>
+int launch_lookup<TRA_FP16>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+template <>
+int launch_lookup<TRA_FP32>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+
+}  // namespace tra
+
+using namespace tra;
+
+struct tra_tbe {
+  int device = 0;
+  int num_features = 0;
+  bool same_dim = true;  // every feature has the same dim (required for POOL_NONE)
+  int dim0 = 0;
+  std::vector<FeatureDesc> slices;  // host copy
+  FeatureDesc* slices_dev = nullptr;
+  int32_t* feats_dev = nullptr;  // all classes' slice lists, concatenated
+  unsigned long long* err_dev = nullptr;
+  std::vector<LaunchClass> classes;
+};
+
+extern "C" {
+
+int tra_version(void) { return 1; }
+
+const char* tra_last_error(void) { return g_err; }
+
+int tra_device_arch(char* buf, int buf_len) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+    set_error("no HIP device");
+    return TRA_ERR_NO_DEVICE;
+  }
+  int dev = 0;
+  TRA_HIP(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  TRA_HIP(hipGetDeviceProperties(&prop, dev));
+  if (buf && buf_len > 0) {
+    strncpy(buf, prop.gcnArchName, (size_t)buf_len - 1);
+    buf[buf_len - 1] = 0;
+  }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error("device arch %s is not gfx950", prop.gcnArchName);
+    return TRA_ERR_NO_DEVICE;
+  }
+  return TRA_OK;
+}
+
+int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
+                   const int32_t* feature_table_map, const int32_t* feature_positions,
+                   int32_t num_features, tra_tbe_t* out) {
+  if (!out || num_tables < 0 || num_features < 0 || (num_tables > 0 && !tables) ||
+      (num_features > 0 && !feature_table_map)) {
+    set_error("tra_tbe_create: null or negative argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  *out = nullptr;
+  for (int t = 0; t < num_tables; ++t) {
+    const tra_table_spec& s = tables[t];
+    const int bits = bits_of(s.dtype);
+    if (bits == 0) {
+      set_error("table %d: unsupported dtype %d", t, s.dtype);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+    if (s.dim <= 0 || s.rows < 0 || (int64_t)s.dim * bits % 32 != 0) {
+      set_error("table %d: dim %d with %d-bit elements is not a whole number of dwords", t,
+                s.dim, bits);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+    const int need = s.dim * bits / 8 + header_bytes(s.dtype);
+    if (s.row_bytes < need || s.row_bytes % 4 != 0 || s.offset % 4 != 0 || s.offset < 0) {
+      set_error("table %d: row_bytes %d (need >= %d) and offset must be multiples of 4", t,
+                s.row_bytes, need);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+  }
+  auto plan = new tra_tbe();
+  plan->num_features = num_features;
+  int col = 0;
+  std::map<std::pair<int, int>, std::vector<int>> by_class;  // (dtype, cb) -> slice ids
+  std::vector<int> slice_lpr;
+  for (int f = 0; f < num_features; ++f) {
+    const int t = feature_table_map[f];
+    if (t < 0 || t >= num_tables || (feature_positions && feature_positions[f] < 0)) {
+      delete plan;
+      set_error("feature %d maps to table %d of %d (or has a negative position)", f, t,
+                num_tables);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+    const tra_table_spec& s = tables[t];
+    if (f == 0) plan->dim0 = s.dim;
+    if (s.dim != plan->dim0) plan->same_dim = false;
+    const int bits = bits_of(s.dtype);
+    const int payload = s.dim * bits / 8;
+    const int cb = payload % 16 == 0 ? 16 : (payload % 8 == 0 ? 8 : 4);
+    const int max_slice = cb * kWaveSize;  // bytes one wave-wide lane group covers
+    for (int off = 0; off < payload; off += max_slice) {
+      const int bytes = std::min(max_slice, payload - off);
+      FeatureDesc d;
+      d.table_offset = s.offset;
+      d.rows = s.rows;
+      d.dim = s.dim;
+      d.row_bytes = s.row_bytes;
+      d.out_col = col + off * 8 / bits;
+      d.dtype = s.dtype;
+      d.feature = feature_positions ? feature_positions[f] : f;
+      d.payload_off = off;
+      by_class[{s.dtype, cb}].push_back((int)plan->slices.size());
+      plan->slices.push_back(d);
+      slice_lpr.push_back(bytes / cb);
+    }
+    col += s.dim;
+  }
+  // Classes: slices sorted by lanes-per-row; at most kMaxSub distinct values each.
+  std::vector<int32_t> all_feats;
+  for (auto& kv : by_class) {
+    std::vector<int>& ids = kv.second;
+    std::stable_sort(ids.begin(), ids.end(),
+                     [&](int x, int y) { return slice_lpr[x] < slice_lpr[y]; });
+    LaunchClass cur;
+    int distinct = 0, last_lpr = -1;
+    auto flush = [&]() {
+      if (!cur.feats.empty()) plan->classes.push_back(cur);
+      cur = LaunchClass();
+      distinct = 0;
+      last_lpr = -1;
+    };
+    for (int id : ids) {
+      if (slice_lpr[id] != last_lpr) {
+        if (distinct == kMaxSub) flush();
+        ++distinct;
+        last_lpr = slice_lpr[id];
+      }
+      cur.dtype = kv.first.first;
+      cur.cb = kv.first.second;
+      cur.feats.push_back(id);
+      cur.lprs.push_back(slice_lpr[id]);
+    }
+    flush();
+  }
+  hipError_t e = hipGetDevice(&plan->device);
+  size_t total = 0;
+  for (auto& c : plan->classes) total += c.feats.size();
+  if (e == hipSuccess && !plan->slices.empty()) {
+    e = hipMalloc((void**)&plan->slices_dev, plan->slices.size() * sizeof(FeatureDesc));
+    if (e == hipSuccess)
+      e = hipMemcpy(plan->slices_dev, plan->slices.data(),
+                    plan->slices.size() * sizeof(FeatureDesc), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc((void**)&plan->feats_dev, total * sizeof(int32_t));
+    if (e == hipSuccess) {
+      size_t pos = 0;
+      for (auto& c : plan->classes) {
+        c.feats_dev = plan->feats_dev + pos;
+        all_feats.insert(all_feats.end(), c.feats.begin(), c.feats.end());
+        pos += c.feats.size();
+      }
+      e = hipMemcpy(plan->feats_dev, all_feats.data(), total * sizeof(int32_t),
+                    hipMemcpyHostToDevice);
+    }
+  }
+  if (e == hipSuccess) e = hipMalloc((void**)&plan->err_dev, sizeof(unsigned long long));
+  if (e == hipSuccess) e = hipMemset(plan->err_dev, 0, sizeof(unsigned long long));
+  if (e != hipSuccess) {
+    tra_tbe_destroy(plan);
+    return hip_fail(e, "tra_tbe_create");
+  }
+  *out = plan;
+  return TRA_OK;
+}
+
+int tra_tbe_destroy(tra_tbe_t tbe) {
+  if (!tbe) return TRA_OK;
+  if (tbe->slices_dev) (void)hipFree(tbe->slices_dev);
+  if (tbe->feats_dev) (void)hipFree(tbe->feats_dev);
+  if (tbe->err_dev) (void)hipFree(tbe->err_dev);
+  delete tbe;
+  return TRA_OK;
+}
+
+int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
+                    const void* offsets, int32_t idx_is_i64, const float* per_sample_weights,
+                    int32_t batch_size, int64_t num_indices, int32_t pooling_mode,
+                    int32_t out_dtype, void* out, int64_t out_stride, void* stream) {
+  if (!tbe) {
+    set_error("tra_tbe_forward: null plan");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (pooling_mode != TRA_POOL_SUM && pooling_mode != TRA_POOL_MEAN &&
+      pooling_mode != TRA_POOL_NONE) {
+    set_error("tra_tbe_forward: bad pooling mode %d", pooling_mode);
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (out_dtype != TRA_FP32 && out_dtype != TRA_FP16) {
+    set_error("tra_tbe_forward: output dtype %d is not fp32/fp16", out_dtype);
+    return TRA_ERR_UNSUPPORTED;
+  }
+  if (batch_size < 0) {
+    set_error("tra_tbe_forward: negative batch size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const bool nobag = pooling_mode == TRA_POOL_NONE;
+  if (tbe->num_features == 0 || batch_size == 0 || (nobag && num_indices == 0)) return TRA_OK;
+  if (!weights || !offsets || !out || (!indices && num_indices != 0)) {
+    set_error("tra_tbe_forward: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (nobag && !tbe->same_dim) {
+    set_error("tra_tbe_forward: sequence lookup needs one embedding dim for all tables");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int esz = out_dtype == TRA_FP16 ? 2 : 4;
+  hipStream_t s = (hipStream_t)stream;
+  for (const LaunchClass& cls : tbe->classes) {
+    LookupArgs a;
+    memset(&a, 0, sizeof(a));
+    a.weights = (const uint8_t*)weights;
+    a.descs = tbe->slices_dev;
+    a.feats = cls.feats_dev;
+    a.indices = indices;
+    a.offsets = offsets;
+    a.psw = nobag ? nullptr : per_sample_weights;
+    a.out = out;
+    a.out_stride = out_stride;
+    a.err_count = tbe->err_dev;
+    a.num_indices = num_indices;
+    a.B = batch_size;
+    a.mean = pooling_mode == TRA_POOL_MEAN;
+    a.out_fp16 = out_dtype == TRA_FP16;
+    const int ne = cls.cb * 8 / bits_of(cls.dtype);
+    bool vec = ((uintptr_t)out % 16 == 0) && ((int64_t)ne * esz % 16 == 0);
+    if (nobag) {
+      vec = vec && ((int64_t)tbe->dim0 * esz % 16 == 0);
+    } else {
+      vec = vec && (out_stride * esz % 16 == 0);
+    }
+    if (!nobag)
+      for (int id : cls.feats) vec = vec && ((int64_t)tbe->slices[id].out_col * esz % 16 == 0);
+    a.vec_store = vec;
+    int grid = 0;
+    int n_sub = 0;
+    for (size_t i = 0; i < cls.feats.size();) {
+      size_t j = i;
+      while (j < cls.feats.size() && cls.lprs[j] == cls.lprs[i]) ++j;
+      SubClass& sc = a.sub[n_sub++];
+      sc.first = (int)i;
+      sc.count = (int)(j - i);
+      sc.lpr = cls.lprs[i];
+      const int per_block = kWavesPerBlock * (kWaveSize / sc.lpr);
+      if (nobag) {
+        // Blocks stride over a feature's ids; enough blocks for ~the average
+        // feature, capped so the grid stays modest.
+        int64_t avg = num_indices > 0 ? num_indices / tbe->num_features + 1 : 4096;
+        int64_t t = (avg + per_block - 1) / per_block;
+        sc.tiles_per_feat = (int)std::max<int64_t>(1, std::min<int64_t>(t, 8192));
+      } else {
+        sc.tiles_per_feat = (batch_size + per_block - 1) / per_block;
+      }
+      sc.tile_start = grid;
+      grid += sc.count * sc.tiles_per_feat;
+      i = j;
+    }
+    a.n_sub = n_sub;
+    int rc;
+    const bool i64 = idx_is_i64 != 0;
+    const bool w = a.psw != nullptr;
+    switch (cls.dtype) {
+      case TRA_INT8: rc = launch_lookup<TRA_INT8>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
+      case TRA_INT4: rc = launch_lookup<TRA_INT4>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
+      case TRA_INT2: rc = launch_lookup<TRA_INT2>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
+      case TRA_FP16: rc = launch_lookup<TRA_FP16>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
+      default: rc = launch_lookup<TRA_FP32>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
+    }
+    if (rc != TRA_OK) return rc;
+  }
+  return TRA_OK;
+}
+
+int tra_tbe_error_count(tra_tbe_t tbe, void* stream, int64_t* count) {
+  if (!tbe || !count) {
+    set_error("tra_tbe_error_count: null argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  unsigned long long v = 0;
+  hipStream_t s = (hipStream_t)stream;
+  TRA_HIP(hipMemcpyAsync(&v, tbe->err_dev, sizeof(v), hipMemcpyDeviceToHost, s));
+  TRA_HIP(hipStreamSynchronize(s));
+  if (v != 0) {
+    TRA_HIP(hipMemsetAsync(tbe->err_dev, 0, sizeof(v), s));
+    TRA_HIP(hipStreamSynchronize(s));
+  }
+  *count = (int64_t)v;
+  return TRA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,765 @@
+"""Sparse containers of the quantized embedding path: JaggedTensor,
+KeyedJaggedTensor (the lookup's input) and KeyedTensor (the pooled output).
+
+Public names, argument order and semantics follow
+torchrec/sparse/jagged_tensor.py (JaggedTensor :562-1030, KeyedJaggedTensor
+:1679-2860, KeyedTensor :3145-3408) for the subset the quantized inference path
+touches: construction, lazily derived lengths <-> offsets, stride, per-key
+totals, split, permute, flatten_lengths, key lookup, to_dict, device moves.
+Variable-stride (VBE) inputs, all-to-all redistribution and pytree / export
+hooks are not part of this package.
+
+Layout: values are feature-major; bag (f, b) is ``lengths[f * B + b]`` long and
+starts at ``offsets[f * B + b]``.  On the GPU, offsets, per-key totals and
+permutation run in the HIP kernels behind ``torchrec_amd.ops``.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple, Union
+
+import torch
+
+from torchrec_amd import ops
+
+
+def _cumsum(o: List[int]) -> List[int]:
+    """Python-list lengths -> offsets (jagged_tensor.py:69-76)."""
+    ret = [0] * (len(o) + 1)
+    for i, x in enumerate(o):
+        ret[i + 1] = ret[i] + x
+    return ret
+
+
+def _to_offsets(lengths: torch.Tensor) -> torch.Tensor:
+    return ops.asynchronous_complete_cumsum(lengths)
+
+
+def _to_lengths(offsets: torch.Tensor) -> torch.Tensor:
+    return torch.diff(offsets)
+
+
+def _maybe_compute_lengths(
+    lengths: Optional[torch.Tensor], offsets: Optional[torch.Tensor]
+) -> torch.Tensor:
+    if lengths is None:
+        assert offsets is not None
+        lengths = _to_lengths(offsets)
+    return lengths
+
+
+def _maybe_compute_offsets(
+    lengths: Optional[torch.Tensor], offsets: Optional[torch.Tensor]
+) -> torch.Tensor:
+    if offsets is None:
+        assert lengths is not None
+        offsets = _to_offsets(lengths)
+    return offsets
+
+
+def _assert_integers(t: Optional[torch.Tensor], name: str) -> None:
+    if t is not None and t.numel() > 0:
+        assert t.dtype in (
+            torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8,
+        ), f"{name} must be of integer type, but got {t.dtype}"
+
+
+def _optional_to(t: Optional[torch.Tensor], device: torch.device, non_blocking: bool):
+    return None if t is None else t.to(device, non_blocking=non_blocking)
+
+
+def _values_string(values: torch.Tensor, start: int, end: int) -> str:
+    size = values.size()
+    if len(size) == 1:
+        return "[" + ", ".join(str(v.item()) for v in values[start:end]) + "]"
+    if len(size) == 2:
+        rows = ["[" + ", ".join(str(v.item()) for v in values[i]) + "]" for i in range(start, end)]
+        return "[" + ", ".join(rows) + "]"
+    raise ValueError("only 1-D or 2-D values can be printed")
+
+
+# ---------------------------------------------------------------------------
+# JaggedTensor
+# ---------------------------------------------------------------------------
+class JaggedTensor:
+    """A batch of variable-length rows stored as one dense ``values`` tensor.
+
+    ``values`` is [N] or [N, D]; ``lengths`` [B] (or ``offsets`` [B + 1])
+    delimit the rows; ``weights`` is an optional per-value tensor.
+    """
+
+    _fields = ["_values", "_weights", "_lengths", "_offsets"]
+
+    def __init__(
+        self,
+        values: torch.Tensor,
+        weights: Optional[torch.Tensor] = None,
+        lengths: Optional[torch.Tensor] = None,
+        offsets: Optional[torch.Tensor] = None,
+    ) -> None:
+        self._values: torch.Tensor = values
+        self._weights: Optional[torch.Tensor] = weights
+        _assert_integers(offsets, "offsets")
+        _assert_integers(lengths, "lengths")
+        assert offsets is not None or lengths is not None, "Must provide lengths or offsets"
+        self._lengths: Optional[torch.Tensor] = lengths
+        self._offsets: Optional[torch.Tensor] = offsets
+
+    @staticmethod
+    def empty(
+        is_weighted: bool = False,
+        device: Optional[torch.device] = None,
+        values_dtype: Optional[torch.dtype] = None,
+        weights_dtype: Optional[torch.dtype] = None,
+        lengths_dtype: torch.dtype = torch.int32,
+    ) -> "JaggedTensor":
+        weights = torch.empty(0, dtype=weights_dtype, device=device) if is_weighted else None
+        return JaggedTensor(
+            values=torch.empty(0, dtype=values_dtype, device=device),
+            offsets=torch.empty(0, dtype=lengths_dtype, device=device),
+            lengths=torch.empty(0, dtype=lengths_dtype, device=device),
+            weights=weights,
+        )
+
+    @staticmethod
+    def from_dense_lengths(
+        values: torch.Tensor, lengths: torch.Tensor, weights: Optional[torch.Tensor] = None
+    ) -> "JaggedTensor":
+        """values [B, N(, D)] padded; row b keeps its first lengths[b] entries."""
+        mask = torch.arange(values.size(1), device=values.device).view(1, -1) < lengths.view(-1, 1)
+        return JaggedTensor(
+            values=values[mask],
+            weights=weights[mask] if weights is not None else None,
+            lengths=lengths,
+        )
+
+    @staticmethod
+    def from_dense(
+        values: List[torch.Tensor], weights: Optional[List[torch.Tensor]] = None
+    ) -> "JaggedTensor":
+        """One tensor per row -> JaggedTensor (offsets kept, lengths derived)."""
+        values_tensor = torch.cat(values, dim=0)
+        lengths = torch.tensor(
+            [v.size(0) for v in values], dtype=torch.int32, device=values_tensor.device
+        )
+        weights_tensor = torch.cat(weights, dim=0) if weights is not None else None
+        return JaggedTensor(values=values_tensor, weights=weights_tensor, lengths=lengths)
+
+    def to_dense(self) -> List[torch.Tensor]:
+        offs = self.offsets().tolist()
+        return [self._values[offs[i] : offs[i + 1]] for i in range(len(offs) - 1)]
+
+    def to_dense_weights(self) -> Optional[List[torch.Tensor]]:
+        if self._weights is None:
+            return None
+        offs = self.offsets().tolist()
+        return [self._weights[offs[i] : offs[i + 1]] for i in range(len(offs) - 1)]
+
+    def to_padded_dense(
+        self, desired_length: Optional[int] = None, padding_value: float = 0.0
+    ) -> torch.Tensor:
+        return self._pad(self._values, desired_length, padding_value)
+
+    def to_padded_dense_weights(
+        self, desired_length: Optional[int] = None, padding_value: float = 0.0
+    ) -> Optional[torch.Tensor]:
+        if self._weights is None:
+            return None
+        return self._pad(self._weights, desired_length, padding_value)
+
+    def _pad(self, data: torch.Tensor, desired_length: Optional[int], padding_value: float):
+        lengths = self.lengths()
+        B = lengths.numel()
+        n = int(lengths.max().item()) if desired_length is None and B else (desired_length or 0)
+        shape = (B, n) + tuple(data.shape[1:])
+        out = data.new_full(shape, padding_value)
+        offs = self.offsets().tolist()
+        for b in range(B):
+            k = min(offs[b + 1] - offs[b], n)
+            out[b, :k] = data[offs[b] : offs[b] + k]
+        return out
+
+    def device(self) -> torch.device:
+        return self._values.device
+
+    def lengths(self) -> torch.Tensor:
+        self._lengths = _maybe_compute_lengths(self._lengths, self._offsets)
+        return self._lengths
+
+    def lengths_or_none(self) -> Optional[torch.Tensor]:
+        return self._lengths
+
+    def offsets(self) -> torch.Tensor:
+        self._offsets = _maybe_compute_offsets(self._lengths, self._offsets)
+        return self._offsets
+
+    def offsets_or_none(self) -> Optional[torch.Tensor]:
+        return self._offsets
+
+    def values(self) -> torch.Tensor:
+        return self._values
+
+    def weights(self) -> torch.Tensor:
+        assert self._weights is not None, "This (Keyed)JaggedTensor doesn't have weights."
+        return self._weights
+
+    def weights_or_none(self) -> Optional[torch.Tensor]:
+        return self._weights
+
+    def to(self, device: torch.device, non_blocking: bool = False) -> "JaggedTensor":
+        return JaggedTensor(
+            values=self._values.to(device, non_blocking=non_blocking),
+            weights=_optional_to(self._weights, device, non_blocking),
+            lengths=_optional_to(self._lengths, device, non_blocking),
+            offsets=_optional_to(self._offsets, device, non_blocking),
+        )
+
+    def record_stream(self, stream: torch.cuda.streams.Stream) -> None:
+        for t in (self._values, self._weights, self._lengths, self._offsets):
+            if t is not None:
+                t.record_stream(stream)
+
+    def __str__(self) -> str:
+        offs = self.offsets().tolist()
+        body = ", ".join(
+            _values_string(self._values, offs[i], offs[i + 1]) for i in range(len(offs) - 1)
+        )
+        return "JaggedTensor({\n    [" + body + "]\n})\n"
+
+
+# ---------------------------------------------------------------------------
+# KeyedJaggedTensor
+# ---------------------------------------------------------------------------
+class KeyedJaggedTensor:
+    """Jagged ids of F named features over a batch of B samples.
+
+    ``keys`` [F]; ``values`` [L] ids; ``lengths`` [F * B] (feature-major) or
+    ``offsets`` [F * B + 1]; ``weights`` optional [L]; ``stride`` = B.
+    """
+
+    _fields = ["_values", "_weights", "_lengths", "_offsets"]
+
+    def __init__(
+        self,
+        keys: List[str],
+        values: torch.Tensor,
+        weights: Optional[torch.Tensor] = None,
+        lengths: Optional[torch.Tensor] = None,
+        offsets: Optional[torch.Tensor] = None,
+        stride: Optional[int] = None,
+        stride_per_key_per_rank: Optional[Union[torch.Tensor, List[List[int]]]] = None,
+        stride_per_key: Optional[List[int]] = None,
+        length_per_key: Optional[List[int]] = None,
+        lengths_offset_per_key: Optional[List[int]] = None,
+        offset_per_key: Optional[List[int]] = None,
+        index_per_key: Optional[Dict[str, int]] = None,
+        jt_dict: Optional[Dict[str, JaggedTensor]] = None,
+        inverse_indices: Optional[Tuple[List[str], torch.Tensor]] = None,
+    ) -> None:
+        if stride_per_key_per_rank is not None or inverse_indices is not None:
+            raise NotImplementedError(
+                "variable-stride (VBE) KeyedJaggedTensors are outside the quantized inference path"
+            )
+        _assert_integers(offsets, "offsets")
+        _assert_integers(lengths, "lengths")
+        self._keys: List[str] = keys
+        self._values: torch.Tensor = values
+        self._weights: Optional[torch.Tensor] = weights
+        self._lengths: Optional[torch.Tensor] = lengths
+        self._offsets: Optional[torch.Tensor] = offsets
+        self._stride: Optional[int] = stride
+        self._stride_per_key: Optional[List[int]] = stride_per_key
+        self._length_per_key: Optional[List[int]] = length_per_key
+        self._offset_per_key: Optional[List[int]] = offset_per_key
+        self._lengths_offset_per_key: Optional[List[int]] = lengths_offset_per_key
+        self._index_per_key: Optional[Dict[str, int]] = index_per_key
+        self._jt_dict: Optional[Dict[str, JaggedTensor]] = jt_dict
+
+    # -- constructors -------------------------------------------------------
+    @staticmethod
+    def from_offsets_sync(
+        keys: List[str],
+        values: torch.Tensor,
+        offsets: torch.Tensor,
+        weights: Optional[torch.Tensor] = None,
+        stride: Optional[int] = None,
+        stride_per_key_per_rank: Optional[List[List[int]]] = None,
+        inverse_indices: Optional[Tuple[List[str], torch.Tensor]] = None,
+    ) -> "KeyedJaggedTensor":
+        kjt = KeyedJaggedTensor(
+            keys=keys, values=values, weights=weights, offsets=offsets, stride=stride,
+            stride_per_key_per_rank=stride_per_key_per_rank, inverse_indices=inverse_indices,
+        )
+        return kjt.sync()
+
+    @staticmethod
+    def from_lengths_sync(
+        keys: List[str],
+        values: torch.Tensor,
+        lengths: torch.Tensor,
+        weights: Optional[torch.Tensor] = None,
+        stride: Optional[int] = None,
+        stride_per_key_per_rank: Optional[List[List[int]]] = None,
+        inverse_indices: Optional[Tuple[List[str], torch.Tensor]] = None,
+    ) -> "KeyedJaggedTensor":
+        kjt = KeyedJaggedTensor(
+            keys=keys, values=values, weights=weights, lengths=lengths, stride=stride,
+            stride_per_key_per_rank=stride_per_key_per_rank, inverse_indices=inverse_indices,
+        )
+        return kjt.sync()
+
+    @staticmethod
+    def empty(
+        is_weighted: bool = False,
+        device: Optional[torch.device] = None,
+        values_dtype: Optional[torch.dtype] = None,
+        weights_dtype: Optional[torch.dtype] = None,
+        lengths_dtype: torch.dtype = torch.int32,
+    ) -> "KeyedJaggedTensor":
+        weights = torch.empty(0, dtype=weights_dtype, device=device) if is_weighted else None
+        return KeyedJaggedTensor(
+            keys=[],
+            values=torch.empty(0, dtype=values_dtype, device=device),
+            weights=weights,
+            lengths=torch.empty(0, dtype=lengths_dtype, device=device),
+            stride=0,
+        )
+
+    @staticmethod
+    def empty_like(kjt: "KeyedJaggedTensor") -> "KeyedJaggedTensor":
+        return KeyedJaggedTensor(
+            keys=[],
+            values=torch.empty(0, device=kjt.device(), dtype=kjt.values().dtype),
+            weights=(
+                None
+                if kjt.weights_or_none() is None
+                else torch.empty(0, device=kjt.device(), dtype=kjt.weights().dtype)
+            ),
+            lengths=torch.empty(0, device=kjt.device(), dtype=kjt.lengths().dtype),
+            stride=kjt.stride(),
+        )
+
+    @staticmethod
+    def from_jt_dict(jt_dict: Dict[str, JaggedTensor]) -> "KeyedJaggedTensor":
+        """All JaggedTensors must share the batch size (same number of lengths)."""
+        keys = list(jt_dict.keys())
+        if not keys:
+            return KeyedJaggedTensor.empty()
+        jts = [jt_dict[k] for k in keys]
+        stride = jts[0].lengths().numel()
+        for jt in jts:
+            assert jt.lengths().numel() == stride, "all features need the same batch size"
+        values = torch.cat([jt.values() for jt in jts])
+        lengths = torch.cat([jt.lengths() for jt in jts])
+        has_w = all(jt.weights_or_none() is not None for jt in jts)
+        weights = torch.cat([jt.weights() for jt in jts]) if has_w else None
+        return KeyedJaggedTensor(
+            keys=keys, values=values, weights=weights, lengths=lengths, stride=stride
+        ).sync()
+
+    @staticmethod
+    def concat(kjt_list: List["KeyedJaggedTensor"]) -> "KeyedJaggedTensor":
+        if not kjt_list:
+            raise ValueError("Can't concat empty KJT list")
+        keys: List[str] = []
+        for k in kjt_list:
+            keys.extend(k.keys())
+        stride = kjt_list[0].stride()
+        weighted = kjt_list[0].weights_or_none() is not None
+        return KeyedJaggedTensor(
+            keys=keys,
+            values=torch.cat([k.values() for k in kjt_list]),
+            weights=torch.cat([k.weights() for k in kjt_list]) if weighted else None,
+            lengths=torch.cat([k.lengths() for k in kjt_list]),
+            stride=stride,
+            length_per_key=[x for k in kjt_list for x in k.length_per_key()],
+        )
+
+    # -- lazily derived state -------------------------------------------------
+    def sync(self) -> "KeyedJaggedTensor":
+        """Materialize the host-side per-key totals now (one small D2H copy)."""
+        self.length_per_key()
+        self.offset_per_key()
+        return self
+
+    def unsync(self) -> "KeyedJaggedTensor":
+        self._length_per_key = None
+        self._offset_per_key = None
+        return self
+
+    def device(self) -> torch.device:
+        return self._values.device
+
+    def lengths(self) -> torch.Tensor:
+        self._lengths = _maybe_compute_lengths(self._lengths, self._offsets)
+        return self._lengths
+
+    def lengths_or_none(self) -> Optional[torch.Tensor]:
+        return self._lengths
+
+    def offsets(self) -> torch.Tensor:
+        self._offsets = _maybe_compute_offsets(self._lengths, self._offsets)
+        return self._offsets
+
+    def offsets_or_none(self) -> Optional[torch.Tensor]:
+        return self._offsets
+
+    def keys(self) -> List[str]:
+        return self._keys
+
+    def values(self) -> torch.Tensor:
+        return self._values
+
+    def weights(self) -> torch.Tensor:
+        assert self._weights is not None, "This (Keyed)JaggedTensor doesn't have weights."
+        return self._weights
+
+    def weights_or_none(self) -> Optional[torch.Tensor]:
+        return self._weights
+
+    def stride(self) -> int:
+        if self._stride is None:
+            nkeys = len(self._keys)
+            if nkeys == 0:
+                self._stride = 0
+            elif self._offsets is not None and self._offsets.numel() > 0:
+                self._stride = (self._offsets.numel() - 1) // nkeys
+            elif self._lengths is not None:
+                self._stride = self._lengths.numel() // nkeys
+            else:
+                self._stride = 0
+        return self._stride
+
+    def stride_per_key(self) -> List[int]:
+        if self._stride_per_key is None:
+            self._stride_per_key = [self.stride()] * len(self._keys)
+        return self._stride_per_key
+
+    def variable_stride_per_key(self) -> bool:
+        return False
+
+    def _key_indices(self) -> Dict[str, int]:
+        if self._index_per_key is None:
+            self._index_per_key = {key: i for i, key in enumerate(self._keys)}
+        return self._index_per_key
+
+    def index_per_key(self) -> Dict[str, int]:
+        return self._key_indices()
+
+    def length_per_key(self) -> List[int]:
+        if self._length_per_key is None:
+            nkeys = len(self._keys)
+            if nkeys == 0:
+                self._length_per_key = []
+            elif self._values.is_meta:
+                total = self._values.numel()
+                lp = [total // nkeys] * nkeys
+                lp[0] += total % nkeys
+                self._length_per_key = lp
+            else:
+                self._length_per_key = ops.length_per_key(self.lengths(), nkeys, self.stride())
+        return self._length_per_key
+
+    def length_per_key_or_none(self) -> Optional[List[int]]:
+        return self._length_per_key
+
+    def offset_per_key(self) -> List[int]:
+        if self._offset_per_key is None:
+            self._offset_per_key = _cumsum(self.length_per_key())
+        return self._offset_per_key
+
+    def offset_per_key_or_none(self) -> Optional[List[int]]:
+        return self._offset_per_key
+
+    def lengths_offset_per_key(self) -> List[int]:
+        if self._lengths_offset_per_key is None:
+            self._lengths_offset_per_key = _cumsum(self.stride_per_key())
+        return self._lengths_offset_per_key
+
+    # -- structure ops -----------------------------------------------------------
+    def split(self, segments: List[int]) -> List["KeyedJaggedTensor"]:
+        """Consecutive groups of segments[i] features each; tensor views, no copies."""
+        out: List[KeyedJaggedTensor] = []
+        start = 0
+        start_offset = 0
+        length_per_key = self.length_per_key()
+        offset_per_key = self.offset_per_key()
+        for segment in segments:
+            end = start + segment
+            end_offset = offset_per_key[end]
+            keys = self._keys[start:end]
+            if segment == len(self._keys):
+                out.append(self)  # whole tensor: no slicing
+            elif segment == 0:
+                dev = self.device()
+                out.append(
+                    KeyedJaggedTensor(
+                        keys=keys,
+                        values=torch.empty(0, device=dev, dtype=self._values.dtype),
+                        weights=(
+                            None
+                            if self._weights is None
+                            else torch.empty(0, device=dev, dtype=self._weights.dtype)
+                        ),
+                        lengths=torch.empty(0, device=dev, dtype=torch.int),
+                        offsets=torch.empty(0, device=dev, dtype=torch.int),
+                        stride=self._stride,
+                    )
+                )
+            else:
+                lo = self.lengths_offset_per_key()
+                out.append(
+                    KeyedJaggedTensor(
+                        keys=keys,
+                        values=self._values[start_offset:end_offset],
+                        weights=(
+                            None if self._weights is None else self._weights[start_offset:end_offset]
+                        ),
+                        lengths=self.lengths()[lo[start] : lo[end]],
+                        stride=self._stride,
+                        length_per_key=length_per_key[start:end],
+                    )
+                )
+            start = end
+            start_offset = end_offset
+        return out
+
+    def permute(
+        self, indices: List[int], indices_tensor: Optional[torch.Tensor] = None
+    ) -> "KeyedJaggedTensor":
+        """New KJT whose feature i is this one's feature indices[i] (repeats allowed)."""
+        if indices_tensor is None:
+            indices_tensor = torch.tensor(indices, dtype=torch.int, device=self.device())
+        length_per_key = self.length_per_key()
+        permuted_keys = [self._keys[i] for i in indices]
+        permuted_length_per_key = [length_per_key[i] for i in indices]
+        total = sum(permuted_length_per_key)
+        permuted_lengths, permuted_values, permuted_weights = ops.permute_2D_sparse_data(
+            indices_tensor,
+            self.lengths().view(len(self._keys), -1),
+            self._values,
+            self._weights,
+            total,
+        )
+        return KeyedJaggedTensor(
+            keys=permuted_keys,
+            values=permuted_values,
+            weights=permuted_weights,
+            lengths=permuted_lengths.view(-1),
+            stride=self._stride,
+            length_per_key=permuted_length_per_key if permuted_keys else None,
+        )
+
+    def flatten_lengths(self) -> "KeyedJaggedTensor":
+        return KeyedJaggedTensor(
+            keys=self._keys,
+            values=self._values,
+            weights=self._weights,
+            lengths=self.lengths().view(-1),
+            stride=self._stride,
+            length_per_key=self.length_per_key(),
+        )
+
+    def __getitem__(self, key: str) -> JaggedTensor:
+        offset_per_key = self.offset_per_key()
+        index = self._key_indices()[key]
+        start = offset_per_key[index]
+        end = offset_per_key[index + 1] if index + 1 < len(offset_per_key) else start
+        lo = self.lengths_offset_per_key()
+        return JaggedTensor(
+            values=self._values[start:end],
+            weights=None if self._weights is None else self._weights[start:end],
+            lengths=self.lengths()[lo[index] : lo[index + 1]],
+        )
+
+    def to_dict(self) -> Dict[str, JaggedTensor]:
+        if self._jt_dict is None:
+            self._jt_dict = {key: self[key] for key in self._keys}
+        return self._jt_dict
+
+    def to(
+        self,
+        device: torch.device,
+        non_blocking: bool = False,
+        dtype: Optional[torch.dtype] = None,
+    ) -> "KeyedJaggedTensor":
+        weights = self._weights
+        if weights is not None:
+            weights = (
+                weights.to(device, dtype=dtype, non_blocking=non_blocking)
+                if dtype is not None
+                else weights.to(device, non_blocking=non_blocking)
+            )
+        return KeyedJaggedTensor(
+            keys=self._keys,
+            values=self._values.to(device, non_blocking=non_blocking),
+            weights=weights,
+            lengths=_optional_to(self._lengths, device, non_blocking),
+            offsets=_optional_to(self._offsets, device, non_blocking),
+            stride=self._stride,
+            stride_per_key=self._stride_per_key,
+            length_per_key=self._length_per_key,
+            lengths_offset_per_key=self._lengths_offset_per_key,
+            offset_per_key=self._offset_per_key,
+            index_per_key=self._index_per_key,
+        )
+
+    def pin_memory(self) -> "KeyedJaggedTensor":
+        pin = lambda t: None if t is None else t.pin_memory()  # noqa: E731
+        return KeyedJaggedTensor(
+            keys=self._keys,
+            values=self._values.pin_memory(),
+            weights=pin(self._weights),
+            lengths=pin(self._lengths),
+            offsets=pin(self._offsets),
+            stride=self._stride,
+            length_per_key=self._length_per_key,
+            offset_per_key=self._offset_per_key,
+        )
+
+    def record_stream(self, stream: torch.cuda.streams.Stream) -> None:
+        for t in (self._values, self._weights, self._lengths, self._offsets):
+            if t is not None:
+                t.record_stream(stream)
+
+    def __str__(self) -> str:
+        if len(self._keys) == 0:
+            return "KeyedJaggedTensor()\n"
+        offs = self.offsets().tolist()
+        B = self.stride()
+        parts = []
+        for f, key in enumerate(self._keys):
+            rows = ", ".join(
+                _values_string(self._values, offs[f * B + b], offs[f * B + b + 1]) for b in range(B)
+            )
+            parts.append(f'    "{key}": [{rows}]')
+        return "KeyedJaggedTensor({\n" + ",\n".join(parts) + "\n})\n"
+
+
+class ComputeKJTToJTDict(torch.nn.Module):
+    """Module form of KeyedJaggedTensor.to_dict (jagged_tensor.py:1320-1361)."""
+
+    def forward(self, keyed_jagged_tensor: KeyedJaggedTensor) -> Dict[str, JaggedTensor]:
+        return keyed_jagged_tensor.to_dict()
+
+
+def jt_is_equal(jt_1: JaggedTensor, jt_2: JaggedTensor) -> bool:
+    if not isinstance(jt_1, JaggedTensor) or not isinstance(jt_2, JaggedTensor):
+        return False
+    if not torch.equal(jt_1.lengths(), jt_2.lengths()):
+        return False
+    if not torch.equal(jt_1.values(), jt_2.values()):
+        return False
+    w1, w2 = jt_1.weights_or_none(), jt_2.weights_or_none()
+    if (w1 is None) != (w2 is None):
+        return False
+    return w1 is None or bool(torch.allclose(w1, w2))
+
+
+def kjt_is_equal(kjt_1: KeyedJaggedTensor, kjt_2: KeyedJaggedTensor) -> bool:
+    if not isinstance(kjt_1, KeyedJaggedTensor) or not isinstance(kjt_2, KeyedJaggedTensor):
+        return False
+    if kjt_1.keys() != kjt_2.keys() or kjt_1.stride() != kjt_2.stride():
+        return False
+    if len(kjt_1.keys()) == 0:
+        return True
+    if not torch.equal(kjt_1.lengths().view(-1), kjt_2.lengths().view(-1)):
+        return False
+    if not torch.equal(kjt_1.values(), kjt_2.values()):
+        return False
+    w1, w2 = kjt_1.weights_or_none(), kjt_2.weights_or_none()
+    if (w1 is None) != (w2 is None):
+        return False
+    return w1 is None or bool(torch.allclose(w1, w2))
+
+
+# ---------------------------------------------------------------------------
+# KeyedTensor
+# ---------------------------------------------------------------------------
+class KeyedTensor:
+    """A dense tensor whose ``key_dim`` is a concatenation of named blocks.
+
+    The pooled lookup returns ``KeyedTensor(keys=embedding names,
+    length_per_key=dims, values=[B, sum(dims)])``.
+    """
+
+    def __init__(
+        self,
+        keys: List[str],
+        length_per_key: List[int],
+        values: torch.Tensor,
+        key_dim: int = 1,
+        offset_per_key: Optional[List[int]] = None,
+        index_per_key: Optional[Dict[str, int]] = None,
+    ) -> None:
+        self._keys = keys
+        self._length_per_key = length_per_key
+        self._values = values
+        self._key_dim = key_dim
+        self._offset_per_key: Optional[List[int]] = offset_per_key
+        self._index_per_key: Optional[Dict[str, int]] = index_per_key
+
+    @staticmethod
+    def from_tensor_list(
+        keys: List[str], tensors: List[torch.Tensor], key_dim: int = 1, cat_dim: int = 1
+    ) -> "KeyedTensor":
+        length_per_key = [t.shape[key_dim] for t in tensors]
+        return KeyedTensor(
+            keys=keys,
+            length_per_key=length_per_key,
+            values=torch.cat(tensors, dim=cat_dim),
+            key_dim=key_dim,
+        )
+
+    def keys(self) -> List[str]:
+        return self._keys
+
+    def values(self) -> torch.Tensor:
+        return self._values
+
+    def key_dim(self) -> int:
+        return self._key_dim
+
+    def device(self) -> torch.device:
+        return self._values.device
+
+    def offset_per_key(self) -> List[int]:
+        if self._offset_per_key is None:
+            self._offset_per_key = _cumsum(self._length_per_key)
+        return self._offset_per_key
+
+    def length_per_key(self) -> List[int]:
+        return self._length_per_key
+
+    def _key_indices(self) -> Dict[str, int]:
+        if self._index_per_key is None:
+            self._index_per_key = {key: i for i, key in enumerate(self._keys)}
+        return self._index_per_key
+
+    def __getitem__(self, key: str) -> torch.Tensor:
+        index = self._key_indices()[key]
+        start = self.offset_per_key()[index]
+        length = self._length_per_key[index]
+        return self._values.narrow(self._key_dim, start, length)
+
+    def to_dict(self) -> Dict[str, torch.Tensor]:
+        pieces = torch.split(self._values, self._length_per_key, dim=self._key_dim)
+        return {key: pieces[i] for i, key in enumerate(self._keys)}
+
+    def to(self, device: torch.device, non_blocking: bool = False) -> "KeyedTensor":
+        return KeyedTensor(
+            keys=self._keys,
+            length_per_key=self._length_per_key,
+            values=self._values.to(device, non_blocking=non_blocking),
+            key_dim=self._key_dim,
+            offset_per_key=self._offset_per_key,
+            index_per_key=self._index_per_key,
+        )
+
+    def record_stream(self, stream: torch.cuda.streams.Stream) -> None:
+        self._values.record_stream(stream)
+
+    def __str__(self) -> str:
+        if len(self._keys) == 0:
+            return "KeyedTensor()\n"
+        parts = [f'    "{k}": {v.tolist()}' for k, v in self.to_dict().items()]
+        return "KeyedTensor({\n" + ",\n".join(parts) + "\n})\n"

@@ -1,0 +1,348 @@
+"""Table-batched quantized embedding operator for MI355X.
+
+``IntNBitTableBatchedEmbeddingBagsCodegen`` keeps the constructor keywords,
+methods and attributes the reference uses from fbgemm_gpu's class of the same
+name (call sites: torchrec/quant/embedding_modules.py:427-438, 461-467,
+547-557, 828-842, 938-942; torchrec/inference/modules.py:628-655; the contract
+as stated by MockTBE, torchrec/distributed/test_utils/infer_utils.py:1037-1096).
+Storage and lookup are this package's own:
+
+* one ``uint8`` buffer per group holds every table; table ``t`` starts at a
+  256-byte aligned offset; a row is ``[fp16 scale][fp16 bias][payload][pad]``
+  for INT8/INT4/INT2 and ``[payload][pad]`` for FP16/FP32, padded to
+  ``row_alignment`` bytes;
+* ``forward`` launches the HIP gather/dequantize/pool kernels of
+  ``libtorchrec_amd.so`` on the current stream.  There is no host lookup: on a
+  CPU device the module can be built, inspected and (de)serialized, but
+  ``forward`` raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+from torch import nn, Tensor
+
+from torchrec_amd import _lib
+from torchrec_amd.tbe.enums import EmbeddingLocation, PoolingMode, SparseType
+
+_SUPPORTED_WEIGHTS = (SparseType.FP32, SparseType.FP16, SparseType.INT8, SparseType.INT4, SparseType.INT2)
+_TABLE_ALIGNMENT = 256
+
+
+def round_up(a: int, b: int) -> int:
+    return (a + b - 1) // b * b
+
+
+def unpadded_row_size_in_bytes(dim: int, weight_ty: SparseType, scale_bias_size_in_bytes: int = 4) -> int:
+    payload = dim * weight_ty.bit_rate() // 8
+    if weight_ty in (SparseType.INT8, SparseType.INT4, SparseType.INT2):
+        return payload + scale_bias_size_in_bytes
+    return payload
+
+
+def rounded_row_size_in_bytes(
+    dim: int, weight_ty: SparseType, row_alignment: int, scale_bias_size_in_bytes: int = 4
+) -> int:
+    return round_up(unpadded_row_size_in_bytes(dim, weight_ty, scale_bias_size_in_bytes), row_alignment)
+
+
+class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
+    """Inference-only table-batched embedding lookup over packed int-N / fp16 rows."""
+
+    def __init__(
+        self,
+        embedding_specs: List[Tuple[str, int, int, SparseType, EmbeddingLocation]],
+        feature_table_map: Optional[List[int]] = None,
+        index_remapping: Optional[List[Tensor]] = None,
+        pooling_mode: PoolingMode = PoolingMode.SUM,
+        device: Optional[torch.device] = None,
+        bounds_check_mode: Optional[int] = None,
+        weight_lists: Optional[List[Tuple[Tensor, Optional[Tensor]]]] = None,
+        output_dtype: SparseType = SparseType.FP16,
+        row_alignment: Optional[int] = None,
+        **unsupported,
+    ) -> None:
+        super().__init__()
+        if index_remapping:
+            raise NotImplementedError("index_remapping (pruning hash maps) is not supported")
+        for k, v in unsupported.items():
+            if v not in (None, False, 0):
+                raise NotImplementedError(f"IntNBitTableBatchedEmbeddingBagsCodegen: option {k}={v!r}")
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else torch.device("cpu")
+        elif not isinstance(device, torch.device):
+            device = torch.device(device)
+        if device.type == "cuda" and device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        self.current_device: torch.device = device
+        self.embedding_specs = embedding_specs
+        self.pooling_mode = pooling_mode
+        self.output_dtype: int = output_dtype.as_int()
+        self.bounds_check_mode_int: int = -1 if bounds_check_mode is None else int(bounds_check_mode)
+        if output_dtype not in (SparseType.FP32, SparseType.FP16):
+            raise NotImplementedError(f"output dtype {output_dtype} (fp32 and fp16 are supported)")
+        self.scale_bias_size_in_bytes = 4
+        self.row_alignment: int = 16 if row_alignment is None else int(row_alignment)
+        if self.row_alignment < 1:
+            raise ValueError("row_alignment must be positive")
+
+        T_ = len(embedding_specs)
+        self.feature_table_map: List[int] = (
+            list(feature_table_map) if feature_table_map is not None else list(range(T_))
+        )
+        assert T_ <= len(self.feature_table_map), "every table needs at least one feature"
+        for t in self.feature_table_map:
+            assert 0 <= t < T_, f"feature_table_map entry {t} out of range"
+        self.embedding_names: List[str] = [e[0] for e in embedding_specs]
+        rows: List[int] = [int(e[1]) for e in embedding_specs]
+        dims: List[int] = [int(e[2]) for e in embedding_specs]
+        self.weight_tys: List[SparseType] = [e[3] for e in embedding_specs]
+        for ty in self.weight_tys:
+            if ty not in _SUPPORTED_WEIGHTS:
+                raise NotImplementedError(f"weight type {ty} (INT8/INT4/INT2/FP16/FP32 are supported)")
+        for name, d, ty in zip(self.embedding_names, dims, self.weight_tys):
+            if (d * ty.bit_rate()) % 32 != 0:
+                raise ValueError(
+                    f"table {name}: embedding_dim {d} at {ty.bit_rate()} bits is not a whole number of 4-byte words"
+                )
+        self.rows = rows
+        self.dims = dims
+        self.max_D: int = max(dims) if dims else 0
+        D_offsets = [0]
+        for t in self.feature_table_map:
+            D_offsets.append(D_offsets[-1] + dims[t])
+        self.D_offsets: List[int] = D_offsets
+        self.total_D: int = D_offsets[-1]
+
+        self.row_bytes: List[int] = []
+        self.weights_physical_offsets: List[int] = []
+        total = 0
+        for r, d, ty in zip(rows, dims, self.weight_tys):
+            rb = rounded_row_size_in_bytes(d, ty, self.row_alignment, self.scale_bias_size_in_bytes)
+            if device.type == "cuda" and rb % 4 != 0:
+                raise ValueError(
+                    f"row_alignment {self.row_alignment} gives {rb}-byte rows; the GPU kernels need a multiple of 4"
+                )
+            self.row_bytes.append(rb)
+            self.weights_physical_offsets.append(total)
+            total = round_up(total + r * rb, _TABLE_ALIGNMENT)
+        self.weights_size: int = total
+        self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
+        self._weights_initialized = False
+        self.weight_initialized = False
+        self.register_buffer("weights_dev", torch.empty(0, dtype=torch.uint8, device=device), persistent=False)
+        if weight_lists is not None:
+            self.initialize_weights()
+            self.assign_embedding_weights(weight_lists)
+
+    # -- storage ------------------------------------------------------------
+    def initialize_weights(self) -> None:
+        if not self._weights_initialized:
+            self.weights_dev = torch.zeros(self.weights_size, dtype=torch.uint8, device=self.current_device)
+            self._weights_initialized = True
+            self.weight_initialized = True
+            self._drop_plan()
+
+    def _rows_view(self, t: int) -> Tensor:
+        off, r, rb = self.weights_physical_offsets[t], self.rows[t], self.row_bytes[t]
+        return self.weights_dev.detach()[off : off + r * rb].view(r, rb)
+
+    def split_embedding_weights_with_scale_bias(
+        self, split_scale_bias_mode: int = 1
+    ) -> List[Tuple[Tensor, Optional[Tensor], Optional[Tensor]]]:
+        """Per-table views that alias the packed buffer.
+
+        mode 0: ``(rows incl. header and padding, None, None)``;
+        mode 1: ``(payload, scale_bias uint8 [rows, 4], None)``;
+        mode 2: ``(payload, scale fp16 [rows, 1], bias fp16 [rows, 1])``.
+        FP16 / FP32 tables have no header: ``(payload, None, None)``.
+        """
+        assert split_scale_bias_mode in (0, 1, 2)
+        if not self._weights_initialized:
+            self.initialize_weights()
+        sb = self.scale_bias_size_in_bytes
+        splits: List[Tuple[Tensor, Optional[Tensor], Optional[Tensor]]] = []
+        for t, ty in enumerate(self.weight_tys):
+            view = self._rows_view(t)
+            if split_scale_bias_mode == 0:
+                splits.append((view, None, None))
+                continue
+            view = view[:, : unpadded_row_size_in_bytes(self.dims[t], ty, sb)]
+            if ty in (SparseType.INT8, SparseType.INT4, SparseType.INT2):
+                if split_scale_bias_mode == 1:
+                    splits.append((view[:, sb:], view[:, :sb], None))
+                else:
+                    splits.append(
+                        (
+                            view[:, sb:],
+                            view[:, : sb // 2].view(torch.float16),
+                            view[:, sb // 2 : sb].view(torch.float16),
+                        )
+                    )
+            else:
+                splits.append((view, None, None))
+        return splits
+
+    def split_embedding_weights(self, split_scale_shifts: bool = True) -> List[Tuple[Tensor, Optional[Tensor]]]:
+        mode = 1 if split_scale_shifts else 0
+        return [(w, s) for (w, s, _) in self.split_embedding_weights_with_scale_bias(mode)]
+
+    def assign_embedding_weights(self, q_weight_list: List[Tuple[Tensor, Optional[Tensor]]]) -> None:
+        """Copy ``(payload, scale_bias)`` per table into the packed buffer."""
+        if not self._weights_initialized:
+            self.initialize_weights()
+        dest = self.split_embedding_weights(split_scale_shifts=True)
+        assert len(q_weight_list) == len(dest), "one (weight, scale_shift) pair per table"
+        if self.current_device.type == "meta":
+            return
+        for (dw, ds), (sw, ss) in zip(dest, q_weight_list):
+            sw = sw.view(torch.uint8) if sw.dtype != torch.uint8 else sw
+            assert dw.shape == sw.shape, f"weight shape {tuple(sw.shape)} != table shape {tuple(dw.shape)}"
+            dw.copy_(sw)
+            if ds is not None:
+                assert ss is not None, "quantized tables need a scale_shift tensor"
+                ss = ss.view(torch.uint8) if ss.dtype != torch.uint8 else ss
+                ds.copy_(ss.reshape(ds.shape))
+
+    # -- lookup -----------------------------------------------------------------
+    def _drop_plan(self) -> None:
+        plans = getattr(self, "_plans", None)
+        if plans:
+            for plan in plans.values():
+                try:
+                    _lib.lib().tra_tbe_destroy(plan)
+                except Exception:  # interpreter shutdown
+                    pass
+            plans.clear()
+
+    def __del__(self) -> None:
+        self._drop_plan()
+
+    def _get_plan(self, feature_positions: Optional[Tuple[int, ...]] = None) -> ctypes.c_void_p:
+        """Launch plan for one placement of the features among the input keys
+        (None: feature f is the f-th key).  Plans are cached per placement."""
+        plan = self._plans.get(feature_positions)
+        if plan is None:
+            T_ = len(self.embedding_specs)
+            specs = (_lib.TableSpec * max(T_, 1))()
+            for t in range(T_):
+                specs[t].offset = self.weights_physical_offsets[t]
+                specs[t].rows = self.rows[t]
+                specs[t].dim = self.dims[t]
+                specs[t].dtype = self.weight_tys[t].as_int()
+                specs[t].row_bytes = self.row_bytes[t]
+            F = len(self.feature_table_map)
+            ftm = (ctypes.c_int32 * max(F, 1))(*self.feature_table_map)
+            pos = None
+            if feature_positions is not None:
+                assert len(feature_positions) == F, "one position per feature"
+                pos = (ctypes.c_int32 * max(F, 1))(*feature_positions)
+            plan = ctypes.c_void_p()
+            with torch.cuda.device(self.current_device):
+                _lib.check(_lib.lib().tra_tbe_create(specs, T_, ftm, pos, F, ctypes.byref(plan)))
+            self._plans[feature_positions] = plan
+        return plan
+
+    def forward(
+        self,
+        indices: Tensor,
+        offsets: Tensor,
+        per_sample_weights: Optional[Tensor] = None,
+        feature_positions: Optional[Sequence[int]] = None,
+        batch_size: Optional[int] = None,
+        out: Optional[Tensor] = None,
+        out_col: int = 0,
+    ) -> Tensor:
+        """Pooled: ``[B, total_D]``; ``PoolingMode.NONE``: ``[indices.numel(), D]``.
+
+        The first three arguments are the reference operator's.  The others let
+        a caller look up straight from a KeyedJaggedTensor whose keys are in a
+        different order (or a superset): ``feature_positions[f]`` is the index
+        of feature ``f`` among the KJT keys, so its bags are
+        ``offsets[feature_positions[f] * B + b]`` with ``B = batch_size``;
+        ``out`` / ``out_col`` make the operator write into columns
+        ``out_col ..`` of a caller-owned ``[B, >= out_col + total_D]`` tensor
+        (``[L, D]`` for PoolingMode.NONE).
+        """
+        dev = self.current_device
+        if dev.type != "cuda":
+            raise _lib.TorchrecAmdError(
+                f"IntNBitTableBatchedEmbeddingBagsCodegen.forward on device {dev}: "
+                "the lookup runs on an MI355X GPU only"
+            )
+        if not self._weights_initialized:
+            raise _lib.TorchrecAmdError("weights are not initialized (call initialize_weights())")
+        _lib.require_gpu(indices, "indices")
+        _lib.require_gpu(offsets, "offsets")
+        if indices.dtype not in (torch.int32, torch.int64):
+            raise TypeError(f"indices must be int32 or int64, got {indices.dtype}")
+        if offsets.dtype != indices.dtype:
+            offsets = offsets.to(indices.dtype)
+        indices = indices.contiguous()
+        offsets = offsets.contiguous()
+        F = len(self.feature_table_map)
+        positions: Optional[Tuple[int, ...]] = None
+        if feature_positions is not None:
+            positions = tuple(int(p) for p in feature_positions)
+            if positions == tuple(range(F)):
+                positions = None
+        if batch_size is None:
+            assert positions is None, "batch_size is required with feature_positions"
+            assert F > 0 and (offsets.numel() - 1) % F == 0, "offsets must have F * B + 1 entries"
+            batch_size = (offsets.numel() - 1) // F
+        B = int(batch_size)
+        n_keys = (max(positions) + 1) if positions else F
+        assert offsets.numel() >= n_keys * B + 1, "offsets shorter than the features it must cover"
+        L = indices.numel()
+        out_dtype = torch.float16 if self.output_dtype == _lib.FP16 else torch.float32
+        nobag = self.pooling_mode == PoolingMode.NONE
+        psw = None
+        if per_sample_weights is not None and not nobag:
+            psw = per_sample_weights.contiguous()
+            if psw.dtype != torch.float32:
+                psw = psw.float()
+            assert psw.numel() == L, "per_sample_weights must have one entry per index"
+        if out is None:
+            shape = (L, self.max_D) if nobag else (B, self.total_D)
+            out = torch.empty(shape, dtype=out_dtype, device=dev)
+            out_col = 0
+        else:
+            assert out.dtype == out_dtype and out.device == dev and out.dim() == 2 and out.stride(1) == 1
+            if nobag:
+                assert out_col == 0 and out.shape[0] >= L and out.shape[1] == self.max_D
+            else:
+                assert out.shape[0] >= B and out.shape[1] >= out_col + self.total_D
+        out_stride = out.stride(0)
+        out_ptr = ctypes.c_void_p(out.data_ptr() + out_col * out.element_size())
+        _lib.check(
+            _lib.lib().tra_tbe_forward(
+                self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices), _lib.ptr(offsets),
+                int(indices.dtype == torch.int64), _lib.ptr(psw), B, L, int(self.pooling_mode),
+                self.output_dtype, out_ptr, out_stride, _lib.current_stream(dev),
+            )
+        )
+        if os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1":
+            bad = self.out_of_range_count()
+            if bad:
+                raise IndexError(f"{bad} embedding indices were out of range")
+        return out
+
+    def out_of_range_count(self) -> int:
+        """Ids outside [0, rows) (other than -1) seen since the last call.  Synchronizes."""
+        total = 0
+        for plan in self._plans.values():
+            n = ctypes.c_int64(0)
+            _lib.check(
+                _lib.lib().tra_tbe_error_count(plan, _lib.current_stream(self.current_device), ctypes.byref(n))
+            )
+            total += int(n.value)
+        return total
+
+    def extra_repr(self) -> str:
+        return (
+            f"tables={len(self.embedding_specs)}, features={len(self.feature_table_map)}, "
+            f"pooling={self.pooling_mode.name}, bytes={self.weights_size}, row_alignment={self.row_alignment}"
+        )
