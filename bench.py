@@ -1,0 +1,465 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized embedding inference path on one MI355X.
+
+Default workload ("c2", the configuration the headline metric is quoted on):
+DLRM-style pooled inference, 26 features / 26 tables, rows log-uniform in
+[1e3, 4e7], dim 128, int4 row-wise with fp16 scale/bias, SUM pooling, fp16
+output, batch 2048, bag lengths U[1, 40] with 5 % forced empty, ids
+Zipf(1.05) over a seeded permutation of each table's rows.  Synthetic, seeded.
+
+A step is one QuantEmbeddingBagCollection.forward over one KeyedJaggedTensor
+(lengths -> offsets scan + the pooled lookup), inputs resident in HBM; steps
+rotate over --batches distinct id batches.  By default each batch's forward is
+captured once in a HIP graph and the timed loop replays the graphs
+(--mode eager times the plain Python calls instead; both are reported).
+
+One JSON line is printed: the metric (pooled lookups/s), the roofline of the
+lookup kernel (algorithmic bytes / HIP-event duration against 8 TB/s) and the
+CPU baseline (fbgemm's own kernels on the host cores, bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=2000)
+    p.add_argument("--warmup", type=int, default=200)
+    p.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    p.add_argument("--batches", type=int, default=8, help="distinct id batches rotated through")
+    p.add_argument("--mode", default="graph", choices=["graph", "eager"])
+    p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline sample")
+    p.add_argument("--scale", type=float, default=1.0, help="shrink table rows (debug only; result is then invalid)")
+    return p.parse_args()
+
+
+# --------------------------------------------------------------------------
+# workloads
+# --------------------------------------------------------------------------
+def zipf_ids(n, rows, alpha, gen, device):
+    """n ids with rank ~ truncated Zipf(alpha) on [1, rows], rank -> id through a seeded permutation."""
+    import torch
+
+    if n == 0:
+        return torch.zeros(0, dtype=torch.int64, device=device)
+    w = torch.arange(1, rows + 1, dtype=torch.float64, device=device).pow_(-alpha)
+    cdf = torch.cumsum(w, 0)
+    cdf /= cdf[-1].clone()
+    u = torch.rand(n, dtype=torch.float64, device=device, generator=gen)
+    rank = torch.searchsorted(cdf, u).clamp_(max=rows - 1)
+    del w, cdf, u
+    perm = torch.randperm(rows, device=device, generator=gen)
+    return perm[rank]
+
+
+def build_workload(args, dev):
+    """Returns dict(module, batches=[(values, lengths, weights)], keys, meta...)."""
+    import numpy as np
+    import torch
+
+    from torchrec_amd import _lib
+    from torchrec_amd.modules.embedding_configs import DataType, EmbeddingBagConfig, EmbeddingConfig, PoolingType
+    from torchrec_amd.quant import EmbeddingBagCollection as QuantEBC, EmbeddingCollection as QuantEC
+
+    cfg = args.config
+    seed = 1000 + int(cfg[1])
+    rng = np.random.default_rng(seed)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    DT = {"int8": DataType.INT8, "int4": DataType.INT4, "int2": DataType.INT2, "fp16": DataType.FP16}
+
+    weighted, pooled, out_dtype, pooling = False, True, torch.half, PoolingType.SUM
+    if cfg == "c1":
+        T, B = 8, 512
+        rows = [100_000] * T
+        dims, dts = [64] * T, ["int8"] * T
+        lens = lambda: np.full(T * B, 20, dtype=np.int64)
+        id_fn = lambda n, r: torch.randint(0, r, (n,), device=dev, generator=gen)
+        desc = "c1: QEBC 8 tables x 100k x 64 int8, B512, L=20, SUM, fp16 out, uniform ids"
+    elif cfg == "c2":
+        T, B = 26, 2048
+        rows = [max(1000, int(round(math.exp(x) * args.scale))) for x in rng.uniform(math.log(1e3), math.log(4e7), T)]
+        dims, dts = [128] * T, ["int4"] * T
+
+        def lens():
+            l = rng.integers(1, 41, T * B)
+            l[rng.random(T * B) < 0.05] = 0
+            return l
+
+        id_fn = lambda n, r: zipf_ids(n, r, 1.05, gen, dev)
+        desc = "c2: QEBC 26 tables rows logU[1e3,4e7] x 128 int4, B2048, len U[1,40] 5% empty, Zipf(1.05), SUM, fp16 out"
+    elif cfg == "c3":
+        T, B = 64, 4096
+        rows = [max(1000, int(round(math.exp(x) * args.scale))) for x in rng.uniform(math.log(1e5), math.log(1e7), T)]
+        dims = [[32, 64, 128, 256][t % 4] for t in range(T)]
+        dts = [["int8", "int4", "int2", "fp16"][(t // 4) % 4] for t in range(T)]
+        lens = lambda: rng.poisson(30, T * B)
+        id_fn = lambda n, r: torch.randint(0, r, (n,), device=dev, generator=gen)
+        weighted, out_dtype = True, torch.float
+        desc = "c3: QEBC 64 tables mixed D{32..256} x {int8,int4,int2,fp16}, B4096, Poisson(30), weighted SUM, fp32 out"
+    elif cfg == "c4":
+        T, B = 16, 1024
+        rows = [max(1000, int(1_000_000 * args.scale))] * T
+        dims, dts = [128] * T, ["int8"] * T
+        lens = lambda: rng.integers(0, 257, T * B)
+        id_fn = lambda n, r: torch.randint(0, r, (n,), device=dev, generator=gen)
+        pooled = False
+        desc = "c4: QEC 16 tables x 1e6 x 128 int8, B1024, len U[0,256], uniform ids, jagged fp16 out"
+    else:
+        T, B = 8, 16384
+        rows = [max(1000, int(250_000_000 * args.scale))] * T
+        dims, dts = [128] * T, ["int4"] * T
+        lens = lambda: np.full(T * B, 80, dtype=np.int64)
+        pooling = PoolingType.MEAN
+        id_fn = None  # affine bijection below: a 250M-entry permutation per table is not needed
+        desc = "c5: QEBC 8 tables x 250M x 128 int4 (68 B rows), B16384, L=80, Zipf(0.8), MEAN, fp16 out"
+
+    if pooled:
+        tables = [
+            EmbeddingBagConfig(name=f"t{t}", embedding_dim=dims[t], num_embeddings=rows[t], feature_names=[f"f{t}"],
+                               data_type=DT[dts[t]], pooling=pooling)
+            for t in range(T)
+        ]
+        module = QuantEBC(tables, weighted, dev, output_dtype=out_dtype, row_alignment=args.row_alignment)
+    else:
+        tables = [
+            EmbeddingConfig(name=f"t{t}", embedding_dim=dims[t], num_embeddings=rows[t], feature_names=[f"f{t}"],
+                            data_type=DT[dts[t]])
+            for t in range(T)
+        ]
+        module = QuantEC(tables, dev, output_dtype=out_dtype, row_alignment=args.row_alignment)
+
+    # Fill the packed store: fp32 N(0, 0.1) rows quantized on the GPU, chunk by chunk,
+    # straight into their header-first rows (c5: synthetic packed bytes, no float master).
+    lib = _lib.lib()
+    stream = _lib.current_stream(dev)
+    BITS = {"int8": 8, "int4": 4, "int2": 2}
+    for tbe in module._emb_modules:
+        for t, name in enumerate(tbe.embedding_names):
+            gt = int(name[1:])
+            view = tbe._rows_view(t)
+            r, rb = tbe.rows[t], tbe.row_bytes[t]
+            step = max(1, (1 << 27) // dims[gt])
+            for r0 in range(0, r, step):
+                n = min(step, r - r0)
+                if cfg == "c5":
+                    chunk = view[r0:r0 + n]
+                    chunk[:, 4:4 + dims[gt] // 2] = torch.randint(0, 256, (n, dims[gt] // 2), dtype=torch.uint8, device=dev, generator=gen)
+                    sc = torch.empty(n, device=dev).uniform_(0.004, 0.02, generator=gen).half()
+                    bi = torch.empty(n, device=dev).uniform_(-0.15, -0.03, generator=gen).half()
+                    chunk[:, 0:2] = sc.view(torch.uint8).view(n, 2)
+                    chunk[:, 2:4] = bi.view(torch.uint8).view(n, 2)
+                    continue
+                w = torch.empty((n, dims[gt]), device=dev).normal_(0, 0.1, generator=gen)
+                if dts[gt] == "fp16":
+                    view[r0:r0 + n, : 2 * dims[gt]] = w.half().view(torch.uint8)
+                else:
+                    dst = tbe.weights_dev.data_ptr() + tbe.weights_physical_offsets[t] + r0 * rb
+                    _lib.check(lib.tra_quantize_rows(_lib.ptr(w), n, dims[gt], BITS[dts[gt]], dst, rb, stream))
+                torch.cuda.synchronize(dev)
+                del w
+
+    batches = []
+    for _ in range(args.batches):
+        l = lens().astype(np.int64)
+        per = l.reshape(T, B).sum(axis=1)
+        if cfg == "c5":
+            vals = []
+            for t in range(T):
+                n, N = int(per[t]), rows[t]
+                # rank ~ truncated Zipf(0.8) by inverse CDF of the continuous envelope, then an affine bijection
+                u = torch.rand(n, dtype=torch.float64, device=dev, generator=gen)
+                a = 1.0 - 0.8
+                rank = ((u * ((N + 1.0) ** a - 1.0) + 1.0).pow_(1.0 / a) - 1.0).long().clamp_(0, N - 1)
+                mul = 2654435761 % N
+                while math.gcd(mul, N) != 1:
+                    mul += 1
+                vals.append((rank * mul + 12345 * (t + 1)) % N)
+            values = torch.cat(vals)
+        else:
+            values = torch.cat([id_fn(int(per[t]), rows[t]) for t in range(T)])
+        values = values.to(torch.int32)
+        lengths = torch.from_numpy(l).to(torch.int32).to(dev)
+        w = torch.rand(values.numel(), device=dev, generator=gen) if weighted else None
+        batches.append((values, lengths, w))
+    torch.cuda.synchronize(dev)
+
+    # algorithmic bytes per call: unpadded rows + ids + weights + offsets + output
+    def alg_bytes(values, lengths):
+        per = lengths.view(T, B).sum(dim=1).tolist()
+        row_b = 0
+        for t in range(T):
+            bits = {"int8": 8, "int4": 4, "int2": 2, "fp16": 16}[dts[t]]
+            row_b += per[t] * (dims[t] * bits // 8 + (4 if dts[t] != "fp16" else 0))
+        L = values.numel()
+        osz = 2 if out_dtype == torch.half else 4
+        out_b = (B * sum(dims) if pooled else L * dims[0]) * osz
+        return row_b + 4 * L + (4 * L if weighted else 0) + 4 * (T * B + 1) + out_b
+
+    return dict(
+        module=module, batches=batches, keys=[f"f{t}" for t in range(T)], T=T, B=B, rows=rows, dims=dims, dts=dts,
+        weighted=weighted, pooled=pooled, out_dtype=out_dtype, desc=desc,
+        alg_bytes=[alg_bytes(v, l) for v, l, _ in batches],
+        store_bytes=sum(m.weights_size for m in module._emb_modules),
+    )
+
+
+# --------------------------------------------------------------------------
+# CPU baseline (fbgemm kernels from libtorch_cpu on the host cores)
+# --------------------------------------------------------------------------
+def cpu_baseline(wl, out_gpu, seconds):
+    import numpy as np
+    import torch
+
+    import oracle as O
+
+    module = wl["module"]
+    tbe = module._emb_modules[0]
+    code = {"fp32": O.FP32, "fp16": O.FP16, "int8": O.INT8, "int4": O.INT4, "int2": O.INT2}
+    values, lengths, w = wl["batches"][0]
+    T, B = wl["T"], wl["B"]
+    ids = values.cpu().numpy()
+    offs = np.zeros(T * B + 1, dtype=np.int32)
+    offs[1:] = np.cumsum(lengths.cpu().numpy())
+    # compact the touched rows so the host never needs the whole store
+    comp_tables, new_ids, pos = [], np.empty_like(ids), 0
+    offsets_t, rows_t, base = [], [], 0
+    pieces = []
+    for t in range(T):
+        seg = ids[offs[t * B]: offs[(t + 1) * B]]
+        uniq, inv = np.unique(seg, return_inverse=True)
+        new_ids[pos:pos + len(seg)] = inv
+        pos += len(seg)
+        rb = tbe.row_bytes[t]
+        view = tbe._rows_view(t)
+        rows = view[torch.from_numpy(uniq.astype(np.int64)).to(view.device)].cpu().numpy() if len(uniq) else np.zeros((0, rb), np.uint8)
+        pieces.append(rows.reshape(-1))
+        offsets_t.append(base)
+        rows_t.append(len(uniq))
+        base += O.round_up(rows.size, 128)
+        pieces.append(np.zeros(base - offsets_t[-1] - rows.size, dtype=np.uint8))
+    store = O.Store(
+        np.concatenate(pieces) if pieces else np.zeros(1, np.uint8),
+        np.asarray(offsets_t, dtype=np.int64), np.asarray(rows_t, dtype=np.int64),
+        np.asarray(tbe.dims, dtype=np.int32), np.asarray([code[str(x)] for x in tbe.weight_tys], dtype=np.int32),
+        np.asarray(tbe.row_bytes, dtype=np.int32),
+    )
+    psw = None if w is None else w.cpu().numpy()
+    pooling = int(tbe.pooling_mode)
+    odt = O.FP16 if wl["out_dtype"] == torch.half else O.FP32
+    nthreads = max(1, min(16, len(os.sched_getaffinity(0))))
+    ftm = list(tbe.feature_table_map)
+    O.tbe_forward(store, ftm, B, new_ids, offs, psw, pooling, odt, "fbgemm", nthreads)  # warm-up / JIT
+    t0, reps = time.perf_counter(), 0
+    while True:
+        ref = O.tbe_forward(store, ftm, B, new_ids, offs, psw, pooling, odt, "fbgemm", nthreads)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > seconds or reps >= 200:
+            break
+    L = ids.size
+    got = out_gpu.cpu().numpy()
+    if not wl["pooled"]:
+        ref = ref[: got.shape[0]]  # rows of the first feature
+    view = np.uint16 if got.dtype == np.float16 else np.uint32
+    mism = int((got.view(view) != ref.view(view)).sum())
+    return {
+        "value": L * reps / el,
+        "unit": "lookups/s",
+        "cores": nthreads,
+        "kind": "reference",
+        "sample": f"batch 0 of the same workload ({L} lookups) x {reps} calls in {el:.1f} s; fbgemm "
+                  f"GenerateEmbeddingSpMDM[NBit]WithStrides from libtorch_cpu, bags split over {nthreads} threads, "
+                  f"tables compacted to the {int(sum(rows_t))} touched rows",
+        "gpu_vs_cpu_mismatching_outputs": mism,
+        "outputs_compared": int(got.size),
+    }
+
+
+# --------------------------------------------------------------------------
+def main():
+    args = parse_args()
+    if args.row_alignment is None:
+        args.row_alignment = 4 if args.config == "c5" else 16
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from torchrec_amd import _lib, KeyedJaggedTensor
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    _lib.lib()  # fail early if the kernel library is missing
+
+    t_setup = time.time()
+    wl = build_workload(args, dev)
+    module, batches, keys = wl["module"], wl["batches"], wl["keys"]
+    NB = len(batches)
+    print(f"[bench] {wl['desc']}; store {wl['store_bytes'] / 1e9:.2f} GB; setup {time.time() - t_setup:.1f} s",
+          file=sys.stderr, flush=True)
+
+    def forward(i):
+        v, l, w = batches[i]
+        return module(KeyedJaggedTensor(keys=keys, values=v, lengths=l, weights=w))
+
+    def out_tensor(o):
+        return o.values() if wl["pooled"] else next(iter(o.values())).values()
+
+    # eager warm-up (creates the launch plans), then optional graph capture
+    outs = [forward(i) for i in range(NB)]
+    torch.cuda.synchronize()
+    graphs = None
+    if args.mode == "graph":
+        graphs, gouts = [], []
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for i in range(NB):
+                forward(i)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        for i in range(NB):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                o = forward(i)
+            graphs.append(g)
+            gouts.append(o)
+        torch.cuda.synchronize()
+        # replays must reproduce the eager result exactly
+        for i in range(NB):
+            graphs[i].replay()
+        torch.cuda.synchronize()
+        for i in range(NB):
+            if not torch.equal(out_tensor(gouts[i]), out_tensor(outs[i])):
+                raise RuntimeError(f"graph replay of batch {i} differs from the eager forward")
+
+    def run(mode, steps):
+        if mode == "graph":
+            for k in range(steps):
+                graphs[k % NB].replay()
+        else:
+            for k in range(steps):
+                forward(k % NB)
+
+    def timed(mode, steps, warmup):
+        run(mode, warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(mode, steps)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    lookups = [b[0].numel() for b in batches]
+    total_lookups = sum(lookups[k % NB] for k in range(args.steps))
+    el = timed(args.mode, args.steps, args.warmup)
+    other = "eager" if args.mode == "graph" else None
+    el_other = timed("eager", args.steps, min(args.warmup, 50)) if other else None
+
+    # ---- kernel-only timing: the lookup launch(es) alone, HIP events on the launch stream
+    tbe = module._emb_modules[0]
+    lib = _lib.lib()
+    offs = []
+    from torchrec_amd import ops
+    for v, l, w in batches:
+        offs.append(ops.asynchronous_complete_cumsum(l))
+    kout = out_tensor(outs[0]).clone()
+    stream = _lib.current_stream(dev)
+    plan = tbe._get_plan(None)
+    pooling = int(tbe.pooling_mode)
+
+    def launch(i):
+        v, l, w = batches[i]
+        rc = lib.tra_tbe_forward(plan, _lib.ptr(tbe.weights_dev), _lib.ptr(v), _lib.ptr(offs[i]), 0, _lib.ptr(w),
+                                 wl["B"], v.numel(), pooling, tbe.output_dtype, _lib.ptr(kout), kout.stride(0), stream)
+        if rc != 0:
+            _lib.check(rc)
+
+    n_launch_per_call = len(module._emb_modules[0]._plans) and 1
+    for k in range(min(args.warmup, 200)):
+        launch(k % NB)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ksteps = args.steps
+    e0.record()
+    for k in range(ksteps):
+        launch(k % NB)
+    e1.record()
+    torch.cuda.synchronize()
+    kernel_ms = e0.elapsed_time(e1) / ksteps
+    alg = sum(wl["alg_bytes"][k % NB] for k in range(ksteps)) / ksteps
+    achieved = alg / (kernel_ms * 1e-3) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"{args.config}_lookup_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    result = {
+        "metric": "pooled lookups/s + achieved HBM GB/s (frac of peak), int4 QuantEBC, 1 GPU",
+        "value": total_lookups / el,
+        "unit": "lookups/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": el / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": wl["desc"],
+            "step": f"QuantEmbeddingBagCollection.forward(KJT) ({args.mode}), {NB} rotating batches",
+            "row_alignment": args.row_alignment,
+            "rows_total": int(sum(wl["rows"])),
+            "store_GB": wl["store_bytes"] / 1e9,
+            "lookups_per_step": sum(lookups) / NB,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": traffic,
+            "kernel": "tbe_pooled_kernel" if wl["pooled"] else "tbe_nobag_kernel",
+            "kernel_ms": kernel_ms,
+            "algorithmic_bytes_per_launch": alg,
+            "kernel_lookups_per_s": (sum(lookups) / NB) / (kernel_ms * 1e-3),
+        },
+    }
+    if other:
+        result["eager_value"] = total_lookups / el_other
+        result["eager_ms_per_step"] = el_other / args.steps * 1e3
+    if not args.no_cpu_baseline:
+        print("[bench] timing the CPU baseline ...", file=sys.stderr, flush=True)
+        result["cpu_baseline"] = cpu_baseline(wl, out_tensor(outs[0]), args.cpu_seconds)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,25 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+def pytest_collection_modifyitems(config, items):
+    # Every GPU test announces itself (flushed) before it touches the device, so a
+    # run that loses the box still names the case that was executing.
+    pass
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    if request.node.get_closest_marker("gpu") is not None:
+        print(f"\n[gpu-case] {request.node.nodeid}", flush=True)
+    yield

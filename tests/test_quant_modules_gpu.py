@@ -1,0 +1,206 @@
+"""QuantEmbeddingBagCollection / QuantEmbeddingCollection end to end on the GPU:
+from_float, key order, shared features, weighted, state_dict round trip.
+Numerics are compared with the CPU oracle fed by the module's own packed store
+(bit-exact), and with the float module at the reference's own loose tolerance
+(atol 0.1, torchrec/quant/tests/test_embedding_modules.py:126)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import bits_equal
+from torchrec_amd import KeyedJaggedTensor
+from torchrec_amd.modules.embedding_configs import DataType, EmbeddingBagConfig, EmbeddingConfig, PoolingType, QuantConfig
+from torchrec_amd.modules.embedding_modules import EmbeddingBagCollection, EmbeddingCollection
+from torchrec_amd.quant.embedding_modules import (
+    _fx_trec_unwrap_kjt,
+    EmbeddingBagCollection as QuantEBC,
+    EmbeddingCollection as QuantEC,
+    quant_prep_enable_quant_state_dict_split_scale_bias,
+)
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+OCODE = {"fp32": O.FP32, "fp16": O.FP16, "int8": O.INT8, "int4": O.INT4, "int2": O.INT2}
+
+
+def oracle_store_of(tbe):
+    """The oracle's view of a module's packed buffer (same bytes, read back from HBM)."""
+    return O.Store(
+        tbe.weights_dev.cpu().numpy(),
+        np.asarray(tbe.weights_physical_offsets, dtype=np.int64),
+        np.asarray(tbe.rows, dtype=np.int64),
+        np.asarray(tbe.dims, dtype=np.int32),
+        np.asarray([OCODE[str(t)] for t in tbe.weight_tys], dtype=np.int32),
+        np.asarray(tbe.row_bytes, dtype=np.int32),
+    )
+
+
+def qconfig(weight_dtype, out_dtype, per_table=None):
+    act = torch.quantization.PlaceholderObserver.with_args(dtype=out_dtype)
+    w = torch.quantization.PlaceholderObserver.with_args(dtype=weight_dtype)
+    return QuantConfig(activation=act, weight=w, per_table_weight_dtype=per_table) if per_table else torch.quantization.QConfig(activation=act, weight=w)
+
+
+def random_kjt(rng, keys, rows, B, max_len, weighted=False, idt=torch.int64):
+    F = len(keys)
+    lengths = rng.integers(0, max_len + 1, F * B)
+    per = lengths.reshape(F, B).sum(axis=1)
+    ids = np.concatenate([rng.integers(0, rows[f], per[f]) for f in range(F)])
+    return KeyedJaggedTensor(
+        keys=list(keys), values=torch.from_numpy(ids).to(idt).to(DEV),
+        lengths=torch.from_numpy(lengths).to(torch.int32).to(DEV),
+        weights=torch.from_numpy(rng.random(len(ids)).astype(np.float32)).to(DEV) if weighted else None)
+
+
+@pytest.mark.parametrize("weight_dtype", [torch.qint8, torch.quint4x2, torch.quint2x4, torch.half])
+@pytest.mark.parametrize("out_dtype", [torch.float, torch.half])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_qebc_from_float(weight_dtype, out_dtype, weighted):
+    rng = np.random.default_rng(0)
+    torch.manual_seed(0)
+    tables = [
+        EmbeddingBagConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1"]),
+        EmbeddingBagConfig(name="t2", embedding_dim=32, num_embeddings=20, feature_names=["f2", "f3"], pooling=PoolingType.MEAN),
+        EmbeddingBagConfig(name="t3", embedding_dim=64, num_embeddings=30, feature_names=["f1"]),
+    ]
+    ebc = EmbeddingBagCollection(tables=tables, is_weighted=weighted, device=DEV)
+    # KJT key order differs from the module's grouped order and has an unused key
+    kjt = random_kjt(rng, ["f3", "unused", "f1", "f2"], [20, 5, 10, 20], B=9, max_len=5, weighted=weighted)
+    want_float = ebc(kjt)
+    ebc.qconfig = qconfig(weight_dtype, out_dtype)
+    qebc = QuantEBC.from_float(ebc)
+    got = qebc(kjt)
+    assert got.values().dtype == out_dtype and got.values().device == DEV
+    # grouped order: SUM tables first (t1, t3), then MEAN (t2)
+    assert got.keys() == ["f1@t1", "f1@t3", "f2", "f3"]
+    assert got.length_per_key() == [16, 64, 32, 32]
+    fl = want_float.to_dict()
+    for k, v in got.to_dict().items():
+        torch.testing.assert_close(v.float(), fl[k].float(), atol=0.1, rtol=0)
+    # oracle on the module's own packed bytes, group by group
+    order = [kjt.keys().index(k) for k in qebc._feature_names]
+    perm = kjt.permute(order)
+    ids, offs = perm.values().cpu().numpy(), perm.offsets().cpu().numpy().astype(np.int64)
+    psw = perm.weights().cpu().numpy() if weighted else None
+    B = kjt.stride()
+    col, f0 = 0, 0
+    gv = got.values().cpu().numpy()
+    for tbe, nf in zip(qebc._emb_modules, qebc._feature_splits):
+        o = offs[f0 * B:(f0 + nf) * B + 1]
+        sl = slice(int(o[0]), int(o[-1]))
+        want = O.tbe_forward(oracle_store_of(tbe), tbe.feature_table_map, B, ids[sl], o - o[0],
+                             None if psw is None else psw[sl], int(tbe.pooling_mode),
+                             O.FP16 if out_dtype == torch.half else O.FP32)
+        assert bits_equal(np.ascontiguousarray(gv[:, col:col + tbe.total_D]), want) == 0
+        col += tbe.total_D
+        f0 += nf
+
+
+def test_qebc_per_table_dtype_and_int32_ids():
+    rng = np.random.default_rng(1)
+    tables = [EmbeddingBagConfig(name=f"t{i}", embedding_dim=d, num_embeddings=50, feature_names=[f"f{i}"])
+              for i, d in enumerate([32, 64, 128, 256])]
+    ebc = EmbeddingBagCollection(tables=tables, device=DEV)
+    ebc.qconfig = qconfig(torch.qint8, torch.half, per_table={"t1": torch.quint4x2, "t2": torch.quint2x4, "t3": torch.half})
+    qebc = QuantEBC.from_float(ebc)
+    assert [str(t) for t in qebc._emb_modules[0].weight_tys] == ["int8", "int4", "int2", "fp16"]
+    assert len(qebc._emb_modules) == 1  # one group although dtypes and dims differ
+    kjt = random_kjt(rng, ["f0", "f1", "f2", "f3"], [50] * 4, B=33, max_len=12, idt=torch.int32)
+    got = qebc(kjt).values().cpu().numpy()
+    tbe = qebc._emb_modules[0]
+    want = O.tbe_forward(oracle_store_of(tbe), [0, 1, 2, 3], 33, kjt.values().cpu().numpy(),
+                         kjt.offsets().cpu().numpy(), None, O.SUM, O.FP16)
+    assert bits_equal(got, want) == 0
+
+
+def test_qebc_state_dict_round_trip():
+    torch.manual_seed(3)
+    mk = lambda: [EmbeddingBagConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1"]),
+                  EmbeddingBagConfig(name="t2", embedding_dim=16, num_embeddings=10, feature_names=["f2"])]
+    for wd in (torch.qint8, torch.quint4x2, torch.quint2x4):
+        for split in (False, True):
+            a = EmbeddingBagCollection(tables=mk(), device=DEV)
+            b = EmbeddingBagCollection(tables=mk(), device=DEV)
+            for m in (a, b):
+                m.qconfig = qconfig(wd, torch.float)
+                if split:
+                    quant_prep_enable_quant_state_dict_split_scale_bias(m)
+            qa, qb = QuantEBC.from_float(a), QuantEBC.from_float(b)
+            kjt = KeyedJaggedTensor(keys=["f1", "f2"], values=torch.tensor([0, 1, 5, 7], device=DEV),
+                                    lengths=torch.tensor([1, 1, 2, 0], device=DEV))
+            assert not torch.equal(qa(kjt).values(), qb(kjt).values())
+            sd = qa.state_dict()
+            assert set(a.state_dict().keys()) <= set(sd.keys())
+            qb.load_state_dict(sd)
+            for k, v in qb.state_dict().items():
+                assert torch.equal(v.view(torch.uint8) if v.dtype == torch.uint8 else v,
+                                   sd[k].view(torch.uint8) if v.dtype == torch.uint8 else sd[k])
+            assert torch.equal(qa(kjt).values(), qb(kjt).values())
+
+
+@pytest.mark.parametrize("weight_dtype", [torch.qint8, torch.quint4x2, torch.half])
+@pytest.mark.parametrize("need_indices", [False, True])
+def test_qec_from_float(weight_dtype, need_indices):
+    rng = np.random.default_rng(2)
+    tables = [EmbeddingConfig(name="t1", embedding_dim=32, num_embeddings=10, feature_names=["f1", "f2"]),
+              EmbeddingConfig(name="t2", embedding_dim=32, num_embeddings=20, feature_names=["f3"])]
+    ec = EmbeddingCollection(tables=tables, device=DEV, need_indices=need_indices)
+    kjt = random_kjt(rng, ["f3", "f1", "x", "f2"], [20, 10, 4, 10], B=7, max_len=6)
+    want_float = ec(kjt)
+    ec.qconfig = qconfig(weight_dtype, torch.half, per_table={"t2": torch.quint4x2} if weight_dtype == torch.qint8 else None)
+    qec = QuantEC.from_float(ec)
+    got = qec(kjt)
+    assert set(got.keys()) == {"f1", "f2", "f3"}
+    jd = kjt.to_dict()
+    for name, jt in got.items():
+        assert jt.values().dtype == torch.half
+        assert torch.equal(jt.lengths(), jd[name].lengths())
+        torch.testing.assert_close(jt.values().float(), want_float[name].values().float(), atol=0.1, rtol=0)
+        if need_indices:
+            assert torch.equal(jt.weights(), jd[name].values())
+        else:
+            assert jt.weights_or_none() is None
+    # oracle, feature by feature
+    f = 0
+    for tbe, nf in zip(qec._emb_modules, qec._feature_splits):
+        store = oracle_store_of(tbe)
+        for k in range(nf):
+            name = qec._feature_names[f]
+            ids = jd[name].values().cpu().numpy()
+            offs = np.array([0, len(ids)], dtype=np.int64)
+            t = tbe.feature_table_map[k]
+            want = O.tbe_forward(store, [t], 1, ids, offs, None, O.NONE, O.FP16)
+            assert bits_equal(got[name].values().cpu().numpy(), want) == 0
+            f += 1
+
+
+def test_qec_shared_feature():
+    rng = np.random.default_rng(8)
+    tables = [EmbeddingConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1"]),
+              EmbeddingConfig(name="t2", embedding_dim=16, num_embeddings=10, feature_names=["f1", "f2"])]
+    ec = EmbeddingCollection(tables=tables, device=DEV)
+    ec.qconfig = qconfig(torch.qint8, torch.float)
+    qec = QuantEC.from_float(ec)
+    kjt = random_kjt(rng, ["f1", "f2"], [10, 10], B=5, max_len=4)
+    got = qec(kjt)
+    want = ec(kjt)
+    assert set(got.keys()) == {"f1@t1", "f1@t2", "f2"}
+    for k in got:
+        torch.testing.assert_close(got[k].values(), want[k].values(), atol=0.1, rtol=0)
+        assert torch.equal(got[k].lengths(), want[k].lengths())
+
+
+def test_unwrap_kjt_dtype_rule_device():
+    kjt = KeyedJaggedTensor(keys=["a"], values=torch.tensor([1, 2], device=DEV), lengths=torch.tensor([2], device=DEV))
+    i, o = _fx_trec_unwrap_kjt(kjt)
+    assert i.dtype == torch.int32 and o.dtype == torch.int32
+
+
+def test_empty_batch_and_empty_features():
+    tables = [EmbeddingBagConfig(name="t", embedding_dim=16, num_embeddings=10, feature_names=["f"], data_type=DataType.INT8)]
+    q = QuantEBC(tables, False, DEV, output_dtype=torch.half)
+    kjt = KeyedJaggedTensor(keys=["f"], values=torch.zeros(0, dtype=torch.int64, device=DEV),
+                            lengths=torch.zeros(4, dtype=torch.int32, device=DEV))
+    out = q(kjt).values()
+    assert out.shape == (4, 16) and not out.any()

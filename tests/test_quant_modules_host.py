@@ -1,0 +1,144 @@
+"""Host-side behaviour of the quantized modules that needs no GPU: grouping,
+naming, key order, dtype mapping, state_dict layout and aliasing, error
+behaviour.  Expectations follow the reference's tests
+(torchrec/quant/tests/test_embedding_modules.py:238-275, 311, 342-402, 849,
+999-1025; torchrec/quant/tests/test_tensor_types.py:24-50)."""
+import pytest
+import torch
+
+from torchrec_amd import _lib, KeyedJaggedTensor
+from torchrec_amd.modules.embedding_configs import (
+    data_type_to_sparse_type,
+    DataType,
+    dtype_to_data_type,
+    EmbeddingBagConfig,
+    EmbeddingConfig,
+    pooling_type_to_pooling_mode,
+    PoolingType,
+)
+from torchrec_amd.modules.embedding_modules import get_embedding_names_by_table
+from torchrec_amd.quant.embedding_modules import (
+    _fx_trec_unwrap_kjt,
+    EmbeddingBagCollection as QuantEBC,
+    EmbeddingCollection as QuantEC,
+)
+from torchrec_amd.tbe import PoolingMode, SparseType
+from torchrec_amd.tensor_types import UInt2Tensor, UInt4Tensor
+
+CPU = torch.device("cpu")
+
+
+def test_dtype_maps():
+    assert dtype_to_data_type(torch.quint4x2) == DataType.INT4
+    assert dtype_to_data_type(torch.quint2x4) == DataType.INT2
+    assert dtype_to_data_type(torch.qint8) == DataType.INT8 == dtype_to_data_type(torch.quint8)
+    assert dtype_to_data_type(torch.uint8) == DataType.UINT8
+    assert dtype_to_data_type(torch.half) == DataType.FP16 and dtype_to_data_type(torch.float) == DataType.FP32
+    assert data_type_to_sparse_type(DataType.UINT8) == SparseType.INT8
+    assert [SparseType.FP32.as_int(), SparseType.FP16.as_int(), SparseType.INT8.as_int(),
+            SparseType.INT4.as_int(), SparseType.INT2.as_int()] == [0, 1, 2, 3, 4]
+    assert pooling_type_to_pooling_mode(PoolingType.MEAN) == PoolingMode.MEAN
+    with pytest.raises(Exception):
+        dtype_to_data_type(torch.complex64)
+
+
+def test_grouping_names_and_order():
+    tables = [
+        EmbeddingBagConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1", "f3"], data_type=DataType.INT4),
+        EmbeddingBagConfig(name="t2", embedding_dim=32, num_embeddings=10, feature_names=["f2"], data_type=DataType.INT8, pooling=PoolingType.MEAN),
+        EmbeddingBagConfig(name="t3", embedding_dim=8, num_embeddings=10, feature_names=["f1"], data_type=DataType.FP16),
+    ]
+    q = QuantEBC(tables, False, CPU, output_dtype=torch.half)
+    # grouped by pooling: SUM tables (t1, t3) first, then MEAN (t2); shared feature f1 gets @table
+    assert [len(m.embedding_specs) for m in q._emb_modules] == [2, 1]
+    assert q._feature_names == ["f1", "f3", "f1", "f2"]
+    assert q._feature_splits == [3, 1]
+    assert q._embedding_names == ["f1@t1", "f3", "f1@t3", "f2"]
+    assert q._length_per_key == [16, 16, 8, 32]
+    assert q._emb_modules[0].pooling_mode == PoolingMode.SUM and q._emb_modules[1].pooling_mode == PoolingMode.MEAN
+    assert get_embedding_names_by_table(tables) == [["f1@t1", "f3"], ["f2"], ["f1@t3"]]
+    assert q.output_dtype() == torch.half and not q.is_weighted() and q.device == CPU
+    with pytest.raises(ValueError, match="Duplicate table name"):
+        QuantEBC([tables[0], tables[0]], False, CPU)
+
+
+def test_ec_dim_mismatch_and_grouping():
+    t = [EmbeddingConfig(name="a", embedding_dim=16, num_embeddings=10, feature_names=["fa"], data_type=DataType.INT8),
+         EmbeddingConfig(name="b", embedding_dim=16, num_embeddings=10, feature_names=["fb"], data_type=DataType.INT4),
+         EmbeddingConfig(name="c", embedding_dim=16, num_embeddings=10, feature_names=["fc"], data_type=DataType.INT8)]
+    q = QuantEC(t, CPU)
+    assert q._feature_names == ["fa", "fc", "fb"] and q._feature_splits == [2, 1]
+    assert q.embedding_names_by_table() == [["fa"], ["fb"], ["fc"]] and q.embedding_dim() == 16
+    with pytest.raises(ValueError, match="same embedding dimension"):
+        QuantEC(t + [EmbeddingConfig(name="d", embedding_dim=8, num_embeddings=10, feature_names=["fd"])], CPU)
+
+
+@pytest.mark.parametrize("split", [False, True])
+def test_state_dict_layout_and_aliasing(split):
+    tables = [
+        EmbeddingBagConfig(name="t8", embedding_dim=16, num_embeddings=10, feature_names=["a"], data_type=DataType.INT8),
+        EmbeddingBagConfig(name="t4", embedding_dim=16, num_embeddings=10, feature_names=["b"], data_type=DataType.INT4),
+        EmbeddingBagConfig(name="t2", embedding_dim=16, num_embeddings=10, feature_names=["c"], data_type=DataType.INT2),
+        EmbeddingBagConfig(name="th", embedding_dim=16, num_embeddings=10, feature_names=["d"], data_type=DataType.FP16),
+    ]
+    q = QuantEBC(tables, False, CPU, quant_state_dict_split_scale_bias=split)
+    sd = q.state_dict()
+    keys = set(sd.keys())
+    assert {f"embedding_bags.{t.name}.weight" for t in tables} <= keys
+    if split:
+        assert {"embedding_bags.t8.weight_qscale", "embedding_bags.t4.weight_qbias"} <= keys
+        assert sd["embedding_bags.t8.weight"].shape == (10, 16)
+        assert sd["embedding_bags.t4.weight"].shape == (10, 16) and isinstance(sd["embedding_bags.t4.weight"], UInt4Tensor)
+        assert sd["embedding_bags.t2.weight"].shape == (10, 16) and isinstance(sd["embedding_bags.t2.weight"], UInt2Tensor)
+        assert sd["embedding_bags.t4.weight"].view(torch.uint8).shape == (10, 8)
+        assert sd["embedding_bags.t8.weight_qscale"].dtype == torch.float16
+        assert sd["embedding_bags.th.weight"].shape == (10, 32)  # fp16 bytes
+    else:
+        assert sd["embedding_bags.t8.weight"].shape == (10, 32)  # 16 + 4 -> padded to 32
+    # buffers alias the packed store: loading a state dict rewrites the store in place
+    tbe = q._emb_modules[0]
+    before = tbe.weights_dev.clone()
+    new_sd = {k: (v.view(torch.uint8).clone() if isinstance(v, (UInt4Tensor, UInt2Tensor)) else v.clone()) for k, v in sd.items()}
+    for k in new_sd:
+        if new_sd[k].dtype == torch.uint8:
+            new_sd[k].fill_(0x5A)
+    wrapped = {}
+    for k, v in new_sd.items():
+        orig = sd[k]
+        wrapped[k] = type(orig)(v) if isinstance(orig, (UInt4Tensor, UInt2Tensor)) else v
+    q.load_state_dict(wrapped)
+    assert not torch.equal(before, tbe.weights_dev)
+    assert (tbe.weights_dev == 0x5A).any()
+
+
+def test_uintx_tensors():
+    e = torch.arange(64, dtype=torch.uint8).view(4, 16)
+    t4 = UInt4Tensor(e)
+    assert t4.shape == (4, 32) and t4.dtype == torch.uint8
+    assert torch.equal(t4.view(torch.uint8), e)
+    assert torch.equal(t4[:, :8].view(torch.uint8), e[:, :4]) and t4[:, :8].shape == (4, 8)
+    assert torch.equal(t4[1:3].view(torch.uint8), e[1:3])
+    t2 = UInt2Tensor(e)
+    assert t2.shape == (4, 64) and torch.equal(t2[:, 8:16].view(torch.uint8), e[:, 2:4])
+    c = t4.clone()
+    assert isinstance(c, UInt4Tensor) and torch.equal(c.view(torch.uint8), e)
+    c.copy_(UInt4Tensor(torch.zeros_like(e)))
+    assert not c.view(torch.uint8).any() and e.any()
+    assert t4.view(8, 16).shape == (8, 16)
+
+
+def test_unwrap_kjt_dtype_rule_host():
+    for dt in (torch.int32, torch.int64):
+        kjt = KeyedJaggedTensor(keys=["a"], values=torch.tensor([1, 2], dtype=dt), lengths=torch.tensor([2], dtype=torch.int32))
+        i, o = _fx_trec_unwrap_kjt(kjt)
+        assert i.dtype == dt and o.dtype == dt
+
+
+def test_forward_without_gpu_fails_loudly():
+    tables = [EmbeddingBagConfig(name="t", embedding_dim=16, num_embeddings=10, feature_names=["f"], data_type=DataType.INT8)]
+    q = QuantEBC(tables, False, CPU)
+    kjt = KeyedJaggedTensor(keys=["f"], values=torch.tensor([1, 2]), lengths=torch.tensor([2]))
+    with pytest.raises(_lib.TorchrecAmdError, match="MI355X"):
+        q(kjt)
+    with pytest.raises(ValueError):  # missing feature
+        q(KeyedJaggedTensor(keys=["g"], values=torch.tensor([1]), lengths=torch.tensor([1])))

@@ -1,0 +1,127 @@
+"""HIP index-math and quantization kernels against the CPU oracle / numpy.
+Integer outputs: torch.equal.  Quantized bytes: identical."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from torchrec_amd import ops
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 65, 4095, 4096, 4097, 100_003, 1_048_577])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_cumsum(n, dtype):
+    rng = np.random.default_rng(n)
+    lengths = rng.integers(0, 50, n).astype(dtype)
+    got = ops.asynchronous_complete_cumsum(torch.from_numpy(lengths).to(DEV)).cpu().numpy()
+    want = O.cumsum(lengths)
+    assert got.dtype == want.dtype and np.array_equal(got, want)
+    assert np.array_equal(want[1:], np.cumsum(lengths, dtype=dtype))  # closed form
+
+
+def test_cumsum_int64_beyond_32_bits():
+    lengths = np.full(5000, 2**31 - 7, dtype=np.int64)
+    got = ops.asynchronous_complete_cumsum(torch.from_numpy(lengths).to(DEV)).cpu().numpy()
+    assert np.array_equal(got[1:], np.cumsum(lengths))
+
+
+@pytest.mark.parametrize("F,B", [(1, 1), (3, 7), (26, 2048), (64, 4096), (5, 300)])
+def test_length_per_key(F, B):
+    rng = np.random.default_rng(F * B)
+    lengths = rng.integers(0, 41, F * B).astype(np.int32)
+    got = ops.length_per_key(torch.from_numpy(lengths).to(DEV), F, B)
+    assert got == lengths.reshape(F, B).sum(axis=1).tolist()
+
+
+@pytest.mark.parametrize("T,B,Tp", [(3, 3, 3), (5, 17, 9), (26, 512, 26), (4, 1000, 2), (2, 1, 6)])
+@pytest.mark.parametrize("idt,vdt,weighted", [(np.int32, np.int64, True), (np.int64, np.int32, False), (np.int32, np.float32, True)])
+def test_permute_2d(T, B, Tp, idt, vdt, weighted):
+    rng = np.random.default_rng(T * 1000 + B + Tp)
+    lengths = rng.integers(0, 9, (T, B)).astype(idt)
+    total = int(lengths.sum())
+    values = rng.integers(0, 10**6, total).astype(vdt)
+    weights = rng.random(total).astype(np.float32) if weighted else None
+    perm = rng.integers(0, T, Tp).astype(np.int32)  # repeats allowed
+    wl, wv, ww = O.permute_2d(perm, lengths, values, weights)
+    gl, gv, gw = ops.permute_2D_sparse_data(
+        torch.from_numpy(perm).to(DEV), torch.from_numpy(lengths).to(DEV), torch.from_numpy(values).to(DEV),
+        None if weights is None else torch.from_numpy(weights).to(DEV))
+    assert np.array_equal(gl.cpu().numpy(), wl)
+    assert np.array_equal(gv.cpu().numpy(), wv)
+    if weighted:
+        assert np.array_equal(gw.cpu().numpy(), ww)
+    else:
+        assert gw is None
+
+
+def _bucketize_python(lengths, ids, weights, block_sizes, W, keep):
+    """Independent pure-Python statement of block bucketization (the same rule as
+    block_bucketize_ref in the reference's torchrec/distributed/tests/test_utils.py:299-466)."""
+    F = len(block_sizes)
+    n = len(lengths)
+    B = n // F
+    buckets = [[[] for _ in range(n)] for _ in range(W)]
+    unb = [-1] * len(ids)
+    j = 0
+    for i in range(n):
+        bs = block_sizes[i // B]
+        for _ in range(lengths[i]):
+            p = ids[j] // bs
+            if p < W:
+                buckets[p][i].append((ids[j] if keep else ids[j] % bs, None if weights is None else weights[j], j))
+            j += 1
+    new_l, new_i, new_w = [], [], []
+    for p in range(W):
+        for i in range(n):
+            new_l.append(len(buckets[p][i]))
+            for v, w, src in buckets[p][i]:
+                unb[src] = len(new_i)
+                new_i.append(v)
+                new_w.append(w)
+    return new_l, new_i, new_w, unb
+
+
+@pytest.mark.parametrize("F,B,W", [(1, 1, 1), (2, 3, 2), (4, 15, 5), (15, 15, 129), (3, 200, 8)])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+@pytest.mark.parametrize("keep", [False, True])
+def test_bucketize(F, B, W, idt, keep):
+    rng = np.random.default_rng(F * 100 + B * 10 + W)
+    lengths = rng.integers(0, 6, F * B).astype(idt)
+    block_sizes = rng.integers(1, 50, F).astype(np.int64)
+    # some ids fall beyond the last bucket and are dropped
+    hi = np.repeat(block_sizes * (W + 1), B)
+    ids = np.concatenate([rng.integers(0, hi[i], lengths[i]) for i in range(F * B)]).astype(idt) if lengths.sum() else np.zeros(0, idt)
+    weights = rng.random(len(ids)).astype(np.float32)
+    pl, pi, pw, pu = _bucketize_python(lengths.tolist(), ids.tolist(), weights.tolist(), block_sizes.tolist(), W, keep)
+    ol, oi, ow, ou = O.bucketize(lengths, ids, block_sizes, W, weights, keep, return_permute=True)
+    assert ol.tolist() == pl and oi.tolist() == pi and ou.tolist() == pu  # oracle pinned by the python rule
+    gl, gi, gw, _, gu = ops.block_bucketize_sparse_features(
+        torch.from_numpy(lengths).to(DEV), torch.from_numpy(ids).to(DEV), False, True,
+        torch.from_numpy(block_sizes).to(DEV), W, torch.from_numpy(weights).to(DEV), keep)
+    assert gl.cpu().numpy().tolist() == pl
+    assert gi.cpu().numpy().tolist() == pi
+    assert gu.cpu().numpy().tolist() == pu
+    assert np.array_equal(gw.cpu().numpy(), np.asarray(pw, dtype=np.float32))
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+def test_quantize_rows_bytes_identical(bits):
+    rng = np.random.default_rng(bits)
+    for dim in (8, 16, 32, 64, 128, 256, 1024):
+        w = rng.normal(0, 0.1, (3000, dim)).astype(np.float32)
+        w[0] = 0.25                                   # constant row: scale 1, all q = 0
+        w[1] = np.linspace(0, 2**bits - 1, dim)       # exact ramp
+        w[2] *= 1e-9                                  # tiny range: fp16 scale underflows
+        w[3] *= 1e4
+        w[4] = 0.0
+        want = O.quantize_sbhalf(w, bits)
+        got = ops.FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(torch.from_numpy(w).to(DEV), bits).cpu().numpy()
+        assert got.shape == want.shape and np.array_equal(got, want), (bits, dim, int((got != want).sum()))
+        # a host tensor is staged through the GPU and comes back on the host
+        got_h = ops.FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(torch.from_numpy(w[:100]), bits)
+        assert got_h.device.type == "cpu" and np.array_equal(got_h.numpy(), want[:100])

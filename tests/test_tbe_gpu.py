@@ -1,0 +1,198 @@
+"""Parity of the HIP lookup (through IntNBitTableBatchedEmbeddingBagsCodegen and
+the C ABI) against the CPU oracle.  The oracle's formula is reproducible
+bit-for-bit and the kernels evaluate it in the same order, so the bar here is
+0 differing bit patterns; that is stricter than the stated tolerance
+(1e-5 relative for fp32 outputs, 2 ulp for fp16 outputs)."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import bits_equal, make_bags, make_table, weight_pair
+from torchrec_amd.tbe import EmbeddingLocation, PoolingMode, SparseType
+from torchrec_amd.tbe.split_table_batched_embeddings_ops_inference import (
+    IntNBitTableBatchedEmbeddingBagsCodegen as TBE,
+)
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+ST = {O.FP32: SparseType.FP32, O.FP16: SparseType.FP16, O.INT8: SparseType.INT8,
+      O.INT4: SparseType.INT4, O.INT2: SparseType.INT2}
+POOL = {O.SUM: PoolingMode.SUM, O.MEAN: PoolingMode.MEAN, O.NONE: PoolingMode.NONE}
+
+
+def build(rng, specs, ftm, pooling, out_dtype, row_alignment):
+    """specs: [(dtype, rows, dim)].  Returns (TBE on GPU, oracle Store)."""
+    datas = [make_table(rng, dt, rows, dim) for dt, rows, dim in specs]
+    store = O.pack_store([(dt, dim, d) for (dt, _, dim), d in zip(specs, datas)], row_alignment=row_alignment)
+    weight_lists = []
+    for (dt, _, _), d in zip(specs, datas):
+        w, sb = weight_pair(dt, d)
+        weight_lists.append((torch.from_numpy(np.ascontiguousarray(w)).to(DEV),
+                             None if sb is None else torch.from_numpy(np.ascontiguousarray(sb)).to(DEV)))
+    tbe = TBE(
+        embedding_specs=[(f"t{i}", rows, dim, ST[dt], EmbeddingLocation.DEVICE) for i, (dt, rows, dim) in enumerate(specs)],
+        feature_table_map=ftm, pooling_mode=POOL[pooling], device=DEV, weight_lists=weight_lists,
+        output_dtype=ST[out_dtype], row_alignment=row_alignment,
+    )
+    return tbe, store
+
+
+def run_both(tbe, store, ftm, B, ids, offsets, psw, pooling, out_dtype):
+    got = tbe(
+        torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV),
+        None if psw is None else torch.from_numpy(psw).to(DEV),
+    ).cpu().numpy()
+    want = O.tbe_forward(store, ftm, B, ids, offsets, psw, pooling, out_dtype)
+    return got, want
+
+
+@pytest.mark.parametrize("dtype", [O.INT8, O.INT4, O.INT2, O.FP16, O.FP32])
+@pytest.mark.parametrize("pooling,weighted", [(O.SUM, False), (O.SUM, True), (O.MEAN, False), (O.MEAN, True), (O.NONE, False)])
+def test_lookup_bit_exact_all_dims(dtype, pooling, weighted):
+    """Every weight type x pooling x {fp32, fp16} out x {int32, int64} ids x dims 32..256,
+    bags 0..80 long with empties, row_alignment 16 and the tight packing."""
+    rng = np.random.default_rng(100 + dtype * 10 + pooling)
+    for dim, out_dtype, idt, align in itertools.product(
+        (32, 64, 128, 256), (O.FP32, O.FP16), (np.int32, np.int64), (16, 4)
+    ):
+        rows, B = 2000, 37
+        specs = [(dtype, rows, dim), (dtype, rows + 13, dim)]
+        ftm = [0, 1, 0]
+        tbe, store = build(rng, specs, ftm, pooling, out_dtype, align)
+        lengths, offsets, ids = make_bags(rng, [rows, rows + 13, rows], B, 80, idt)
+        psw = rng.uniform(-1, 1, len(ids)).astype(np.float32) if weighted else None
+        got, want = run_both(tbe, store, ftm, B, ids, offsets, psw, pooling, out_dtype)
+        assert bits_equal(got, want) == 0, (dim, out_dtype, idt, align)
+        assert tbe.out_of_range_count() == 0
+
+
+def test_mixed_group_one_call():
+    """One TBE group mixing all weight types and dims 32/64/128/256 (weighted SUM, fp32 out)."""
+    rng = np.random.default_rng(3)
+    specs = []
+    for t in range(16):
+        specs.append(([O.INT8, O.INT4, O.INT2, O.FP16][(t // 4) % 4], 500 + 7 * t, [32, 64, 128, 256][t % 4]))
+    ftm = list(range(16))
+    tbe, store = build(rng, specs, ftm, O.SUM, O.FP32, 16)
+    B = 64
+    lengths, offsets, ids = make_bags(rng, [s[1] for s in specs], B, 40)
+    psw = rng.uniform(0, 1, len(ids)).astype(np.float32)
+    got, want = run_both(tbe, store, ftm, B, ids, offsets, psw, O.SUM, O.FP32)
+    assert bits_equal(got, want) == 0
+    # stated tolerance, for the record
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize("dtype,dim", [(O.INT8, 8), (O.INT8, 12), (O.INT8, 24), (O.INT4, 8), (O.INT4, 24),
+                                       (O.INT4, 40), (O.INT2, 16), (O.INT2, 48), (O.FP16, 2), (O.FP16, 6),
+                                       (O.FP16, 20), (O.FP32, 1), (O.FP32, 3), (O.FP32, 10), (O.INT8, 1040),
+                                       (O.FP16, 1000), (O.FP32, 520)])
+def test_odd_dims(dtype, dim):
+    """Payloads that are not multiples of 16 bytes (8- and 4-byte lane chunks) and
+    rows wider than one wave of 16-byte chunks (column slices)."""
+    rng = np.random.default_rng(dim)
+    for pooling in (O.SUM, O.NONE):
+        rows, B = 300, 19
+        tbe, store = build(rng, [(dtype, rows, dim)], [0], pooling, O.FP32, 4)
+        lengths, offsets, ids = make_bags(rng, [rows], B, 9)
+        got, want = run_both(tbe, store, [0], B, ids, offsets, None, pooling, O.FP32)
+        assert bits_equal(got, want) == 0
+
+
+def test_edge_bags():
+    """All-empty input, a single very long bag, pruned ids (-1), and out-of-range ids."""
+    rng = np.random.default_rng(11)
+    rows, dim, B = 1000, 128, 8
+    tbe, store = build(rng, [(O.INT4, rows, dim)], [0], O.SUM, O.FP16, 16)
+    # all bags empty -> exact zeros
+    offsets = np.zeros(B + 1, dtype=np.int32)
+    ids = np.zeros(0, dtype=np.int32)
+    got, want = run_both(tbe, store, [0], B, ids, offsets, None, O.SUM, O.FP16)
+    assert bits_equal(got, want) == 0 and not got.any()
+    # one bag of 5000 ids, the rest empty
+    offsets = np.zeros(B + 1, dtype=np.int32)
+    offsets[4:] = 5000
+    ids = rng.integers(0, rows, 5000).astype(np.int32)
+    got, want = run_both(tbe, store, [0], B, ids, offsets, None, O.SUM, O.FP16)
+    assert bits_equal(got, want) == 0
+    # -1 ids are skipped, exactly as the CPU kernels do
+    ids2 = ids.copy()
+    ids2[::7] = -1
+    got, want = run_both(tbe, store, [0], B, ids2, offsets, None, O.SUM, O.FP16)
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
+    # ids >= rows are skipped and counted
+    ids3 = ids.copy()
+    ids3[:5] = rows + 3
+    got = tbe(torch.from_numpy(ids3).to(DEV), torch.from_numpy(offsets).to(DEV)).cpu().numpy()
+    ids3[:5] = -1
+    want = O.tbe_forward(store, [0], B, ids3, offsets, None, O.SUM, O.FP16)
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 5
+    assert tbe.out_of_range_count() == 0
+
+
+def test_feature_positions_and_out_columns():
+    """Lookup straight from a key order that differs from the operator's features,
+    with an unused key in between, writing into a slice of a wider output."""
+    rng = np.random.default_rng(5)
+    rows, dim, B = 800, 64, 33
+    specs = [(O.INT8, rows, dim), (O.INT4, rows, dim)]
+    tbe, store = build(rng, specs, [0, 1], O.SUM, O.FP32, 16)
+    # KJT keys: [f1, unused, f0]
+    lengths, offsets, ids = make_bags(rng, [rows, rows, rows], B, 20)
+    out = torch.full((B, 3 * dim + 5), 7.0, device=DEV)
+    tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV), feature_positions=[2, 0],
+        batch_size=B, out=out, out_col=dim)
+    # oracle: reorder by hand
+    seg = [ids[offsets[k * B]:offsets[(k + 1) * B]] for k in range(3)]
+    L = lengths.reshape(3, B)
+    o_len = np.concatenate([L[2], L[0]])
+    o_off = np.zeros(2 * B + 1, dtype=np.int32)
+    o_off[1:] = np.cumsum(o_len)
+    want = O.tbe_forward(store, [0, 1], B, np.concatenate([seg[2], seg[0]]), o_off, None, O.SUM, O.FP32)
+    got = out.cpu().numpy()
+    assert bits_equal(np.ascontiguousarray(got[:, dim:3 * dim]), want) == 0
+    assert (got[:, :dim] == 7.0).all() and (got[:, 3 * dim:] == 7.0).all()
+
+
+def test_config1_shape_full():
+    """BASELINE config 1 at full size: 8 tables x 100k x 64 int8, B=512, L=20, SUM, fp16 out."""
+    rng = np.random.default_rng(1001)
+    T, rows, dim, B = 8, 100_000, 64, 512
+    specs = [(O.INT8, rows, dim)] * T
+    tbe, store = build(rng, specs, list(range(T)), O.SUM, O.FP16, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 20, fixed_len=20)
+    got, want = run_both(tbe, store, list(range(T)), B, ids, offsets, None, O.SUM, O.FP16)
+    assert got.shape == (512, 512)
+    assert bits_equal(got, want) == 0
+
+
+def test_properties_large():
+    """Size-independent properties on a larger problem (no oracle run):
+    weighted with w == 1 equals unweighted; MEAN == SUM * (1/len) in fp32;
+    permuting features permutes output columns only."""
+    rng = np.random.default_rng(77)
+    T, rows, dim, B = 12, 200_000, 128, 2048
+    specs = [(O.INT4, rows, dim)] * T
+    datas = [make_table(rng, O.INT4, rows, dim) for _ in range(T)]
+    wl = [(torch.from_numpy(np.ascontiguousarray(d[:, :-4])).to(DEV), torch.from_numpy(np.ascontiguousarray(d[:, -4:])).to(DEV)) for d in datas]
+    mk = lambda pooling, order: TBE(
+        embedding_specs=[(f"t{i}", rows, dim, SparseType.INT4, EmbeddingLocation.DEVICE) for i in order],
+        pooling_mode=pooling, device=DEV, weight_lists=[wl[i] for i in order], output_dtype=SparseType.FP32)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 40)
+    ti, to = torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV)
+    s = mk(PoolingMode.SUM, range(T))
+    a = s(ti, to)
+    b = s(ti, to, torch.ones(len(ids), device=DEV))
+    assert torch.equal(a, b)
+    m = mk(PoolingMode.MEAN, range(T))(ti, to)
+    ln = torch.from_numpy(lengths.astype(np.int64)).to(DEV).view(T, B).t().float()  # [B, T]
+    inv = torch.where(ln > 0, 1.0 / ln, torch.ones_like(ln)).repeat_interleave(dim, dim=1)
+    assert torch.equal(m, a * inv)
+    order = list(rng.permutation(T))
+    p = mk(PoolingMode.SUM, order)(ti, to, feature_positions=order, batch_size=B)
+    assert torch.equal(p.view(B, T, dim), a.view(B, T, dim)[:, order, :])
