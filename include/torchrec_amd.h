@@ -98,7 +98,7 @@ int tra_tbe_destroy(tra_tbe_t tbe);
  *   out          device; pooled: [B, out_stride] elements, feature f at column
  *                D_offsets[f]; TRA_POOL_NONE: [L, dim] (all features share dim)
  *   out_dtype    TRA_FP32 or TRA_FP16
- *   num_indices  L (sizes the TRA_POOL_NONE launch; pass -1 if unknown)
+ *   num_indices  L, the number of elements of indices (required)
  * Arithmetic per output column, ids in order: acc = fmaf(w*scale, q, acc +
  * w*bias) (fp16/fp32 rows: acc = fmaf(w, x, acc)); MEAN multiplies by 1.0f/len;
  * output rounded to nearest even.  Ids outside [0, rows) other than -1 are

@@ -50,6 +50,11 @@ struct LookupArgs {
   int32_t mean;
   int32_t vec_store;  // 1: every lane's output slice is 16-byte aligned
   int32_t out_fp16;
+  int32_t window_bags;  // balanced pooled kernel: bags per block
+  int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
+#ifdef TRA_INSTRUMENT
+  unsigned long long* ts;  // [waves][8] wall-clock stamps
+#endif
   SubClass sub[kMaxSub];
 };
 
@@ -184,48 +189,80 @@ struct RowBuf {
   int valid;  // 1: accumulate; 0: skip
 };
 
-template <int DTYPE, int CB, typename IdxT, bool WEIGHTED>
-__device__ __forceinline__ void fetch_row(RowBuf<CB>& r, bool in_range, int64_t j,
-                                          const LookupArgs& a, const uint8_t* table,
-                                          int64_t rows, int64_t row_bytes,
-                                          int chunk_off, bool count_errors) {
-  r.valid = 0;
-  r.hdr = 0;
-  r.w = 1.0f;
-  if (in_range) {
-    const int64_t id = load_index<IdxT>(a.indices, j);
-    if ((uint64_t)id < (uint64_t)rows) {
-      const uint8_t* row = table + id * row_bytes;
-      if constexpr (Traits<DTYPE>::kHeader != 0)
-        r.hdr = *reinterpret_cast<const uint32_t*>(row);
-      r.d = load_chunk<CB>(row + chunk_off);
-      if constexpr (WEIGHTED) r.w = a.psw[j];
-      r.valid = 1;
-    } else if (id != -1 && count_errors) {
-      atomicAdd(a.err_count, 1ull);
-    }
-  }
+// Id of position j, or -1 (= skip) when the position is outside the bag.  The
+// load itself is unconditional (position clamped into the ids array) and the
+// result is selected afterwards: a load under a lane predicate would be
+// followed by a full wait at the re-convergence point and serialize the ids.
+template <typename IdxT>
+__device__ __forceinline__ int64_t fetch_id(const LookupArgs& a, bool in_range, int64_t j) {
+  const int64_t jc = j < a.num_indices ? j : a.num_indices - 1;
+  const int64_t id = load_index<IdxT>(a.indices, jc);
+  return in_range ? id : (int64_t)-1;
 }
 
+// Issue the loads of one row chunk (header dword, CB payload bytes, weight).
+// Branch-free: an id outside [0, rows) (a pruned id -1, a lane past the end of
+// its bag, or a bad id) is redirected to row 0 and flagged invalid; consume_row
+// then multiplies it away exactly.  Returns 1 for a bad id (out of range and
+// not -1).
+template <int DTYPE, int CB, bool WEIGHTED>
+__device__ __forceinline__ int fetch_row(RowBuf<CB>& r, int64_t id, int64_t j,
+                                          const LookupArgs& a, const uint8_t* lane_base,
+                                          int64_t rows, int64_t row_bytes, int chunk_off) {
+  const bool valid = (uint64_t)id < (uint64_t)rows;
+  const int64_t idc = valid ? id : 0;
+  const uint8_t* chunk = lane_base + idc * row_bytes;  // lane_base = table + chunk_off
+#ifdef TRA_EXP_NO_ROW_LOADS
+  r.hdr = 0x3c003c00u;
+#pragma unroll
+  for (int i = 0; i < CB / 4; ++i) r.d.v[i] = (uint32_t)id * 2654435761u + i;
+#else
+  if constexpr (Traits<DTYPE>::kHeader != 0)
+    r.hdr = *reinterpret_cast<const uint32_t*>(chunk - chunk_off);
+  else
+    r.hdr = 0;
+  r.d = load_chunk<CB>(chunk);
+#endif
+  if constexpr (WEIGHTED) {
+    const int64_t jc = j < a.num_indices ? j : a.num_indices - 1;
+    r.w = a.psw[jc];
+  } else {
+    r.w = 1.0f;
+  }
+  r.valid = valid;
+  return (!valid && id != -1) ? 1 : 0;
+}
+
+// Accumulate one fetched row chunk.  An invalid row contributes fmaf(+0, q,
+// acc + (+0)), which leaves acc unchanged bit-for-bit: acc is never -0 (it
+// starts at +0 and a round-to-nearest sum is -0 only if both addends are), and
+// q is a finite integer.  For fp16 / fp32 rows the payload of an invalid row is
+// zeroed as well, so a stored inf / nan in row 0 cannot leak in.
 template <int DTYPE, int CB, bool WEIGHTED>
 __device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r) {
-  if (r.valid) {
-    float s, b;
-    if constexpr (Traits<DTYPE>::kHeader != 0) {
-      s = half_bits_to_float(r.hdr & 0xffffu);
-      b = half_bits_to_float(r.hdr >> 16);
-      if constexpr (WEIGHTED) {
-        s = r.w * s;
-        b = r.w * b;
-      }
-    } else {
-      s = r.w;
-      b = 0.0f;
+#ifdef TRA_EXP_NO_DEQUANT
+  acc[0] += __builtin_bit_cast(float, r.d.v[0] ^ r.d.v[CB / 4 - 1] ^ r.hdr);
+  return;
+#endif
+  constexpr int EPD = 32 / Traits<DTYPE>::kBits;  // elements per dword
+  float s, b;
+  if constexpr (Traits<DTYPE>::kHeader != 0) {
+    s = half_bits_to_float(r.hdr & 0xffffu);
+    b = half_bits_to_float(r.hdr >> 16);
+    if constexpr (WEIGHTED) {
+      s = r.w * s;
+      b = r.w * b;
     }
-    constexpr int EPD = 32 / Traits<DTYPE>::kBits;  // elements per dword
+    s = r.valid ? s : 0.0f;
+    b = r.valid ? b : 0.0f;
 #pragma unroll
     for (int i = 0; i < CB / 4; ++i)
       accumulate_dword<DTYPE, WEIGHTED>(acc + i * EPD, r.d.v[i], s, b);
+  } else {
+    s = r.valid ? r.w : 0.0f;
+#pragma unroll
+    for (int i = 0; i < CB / 4; ++i)
+      accumulate_dword<DTYPE, WEIGHTED>(acc + i * EPD, r.valid ? r.d.v[i] : 0u, s, 0.0f);
   }
 }
 
@@ -297,10 +334,95 @@ __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lp
   return true;
 }
 
-// ---- pooled lookup: one lane group per bag --------------------------------
+#ifdef TRA_INSTRUMENT
+#define TRA_STAMP(k)                                                                      \
+  do {                                                                                    \
+    if ((threadIdx.x & 63) == 0)                                                          \
+      a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64) * 8 + (k)] = wall_clock64(); \
+  } while (0)
+#else
+#define TRA_STAMP(k)
+#endif
+
+// ---- pooled lookup ----------------------------------------------------------
+// Everything a lane needs to walk rows of its feature's table.
+struct RowWalk {
+  const uint8_t* lane_base;  // table + this lane's chunk offset inside a row
+  int64_t rows;
+  int64_t row_bytes;
+  int chunk_off;
+  bool count_errors;
+};
+
+// Pool one bag per lane group: ids [start, start + len), in order, into acc.
+// max_len is the longest bag among the wave's lane groups (wave-uniform trip
+// count).  Software pipeline, per lane group: ids are requested two batches of
+// U rows ahead, row chunks one batch ahead, so neither an id load nor a row
+// load is waited for in the batch that issued it.
+template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, int NE>
+__device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
+                                         const RowWalk& w, int64_t start, int len,
+                                         int max_len_any_lane) {
+  // Wave-uniform by construction; telling the compiler keeps the loop control
+  // on the scalar unit and the loads free of lane-mask bookkeeping.
+  const int max_len = __builtin_amdgcn_readfirstlane(max_len_any_lane);
+  int64_t idA[U], idB[U];
+  RowBuf<CB> bufA[U], bufB[U];
+  int bad = 0;
+  // Row slots at or beyond max_len belong to no lane group: the (wave-uniform)
+  // tests below skip their loads and their arithmetic altogether.
+#pragma unroll
+  for (int u = 0; u < U; ++u) idA[u] = fetch_id<IdxT>(a, u < len, start + u);
+#pragma unroll
+  for (int u = 0; u < U; ++u) idB[u] = fetch_id<IdxT>(a, U + u < len, start + U + u);
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    bad += fetch_row<DTYPE, CB, WEIGHTED>(bufA[u], idA[u], start + u, a, w.lane_base, w.rows,
+                                          w.row_bytes, w.chunk_off);
+  for (int it = 0; it < max_len; it += 2 * U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      idA[u] = fetch_id<IdxT>(a, it + 2 * U + u < len, start + it + 2 * U + u);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      bad += fetch_row<DTYPE, CB, WEIGHTED>(bufB[u], idB[u], start + it + U + u, a, w.lane_base,
+                                            w.rows, w.row_bytes, w.chunk_off);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (it + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufA[u]);
+    if (it + U >= max_len) break;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      idB[u] = fetch_id<IdxT>(a, it + 3 * U + u < len, start + it + 3 * U + u);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      bad += fetch_row<DTYPE, CB, WEIGHTED>(bufA[u], idA[u], start + it + 2 * U + u, a,
+                                            w.lane_base, w.rows, w.row_bytes, w.chunk_off);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (it + U + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
+  }
+  // Bad ids are counted by the lane that owns column 0.
+  if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
+}
+
+template <int NE>
+__device__ __forceinline__ void finish_bag(float (&acc)[NE], const LookupArgs& a, int len,
+                                           int64_t pos) {
+  if (a.mean && len > 0) {
+    const float inv = 1.0f / (float)len;
+#pragma unroll
+    for (int i = 0; i < NE; ++i) acc[i] *= inv;
+  }
+  store_outputs<NE>(a, pos, acc);
+}
+
+// Static mapping: lane group g of wave w of tile t owns bag (t*waves + w)*gpw + g.
+// Used for small problems, where there are not enough bags to balance.
 template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U>
 __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;  // columns per lane
+  TRA_STAMP(0);
   int f, lpr, tile;
   if (!locate_tile(a, f, lpr, tile)) return;
   const FeatureDesc d = a.descs[f];
@@ -320,47 +442,153 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
   }
   const int len = (int)(end - start);
   const int max_len = wave_max(len);
+  TRA_STAMP(1);
 
-  const uint8_t* table = a.weights + d.table_offset;
-  const int chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
-  const int64_t rows = d.rows;
-  const int64_t row_bytes = d.row_bytes;
-  const bool count_errors = c == 0 && d.payload_off == 0;
+  RowWalk w;
+  w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
+  w.lane_base = a.weights + d.table_offset + w.chunk_off;
+  w.rows = d.rows;
+  w.row_bytes = d.row_bytes;
+  w.count_errors = c == 0 && d.payload_off == 0;
 
   float acc[NE];
 #pragma unroll
   for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
-
-  RowBuf<CB> bufA[U], bufB[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u)
-    fetch_row<DTYPE, CB, IdxT, WEIGHTED>(bufA[u], u < len, start + u, a, table, rows,
-                                          row_bytes, chunk_off, count_errors);
-  for (int it = 0; it < max_len; it += 2 * U) {
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      fetch_row<DTYPE, CB, IdxT, WEIGHTED>(bufB[u], it + U + u < len, start + it + U + u,
-                                            a, table, rows, row_bytes, chunk_off, count_errors);
-#pragma unroll
-    for (int u = 0; u < U; ++u) consume_row<DTYPE, CB, WEIGHTED>(acc, bufA[u]);
-    if (it + U >= max_len) break;
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      fetch_row<DTYPE, CB, IdxT, WEIGHTED>(bufA[u], it + 2 * U + u < len,
-                                            start + it + 2 * U + u, a, table, rows,
-                                            row_bytes, chunk_off, count_errors);
-#pragma unroll
-    for (int u = 0; u < U; ++u) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
-  }
-
+  pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+  TRA_STAMP(2);
+#ifdef TRA_INSTRUMENT
+  if ((threadIdx.x & 63) == 0)
+    a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64) * 8 + 4] = max_len;
+#endif
   if (!active) return;
-  if (a.mean && len > 0) {
-    const float inv = 1.0f / (float)len;
+  finish_bag<NE>(acc, a, len,
+                 (int64_t)bag_in_feat * a.out_stride + d.out_col + (int64_t)c * NE);
+  TRA_STAMP(3);
+}
+
+// Balanced mapping.  One 1024-thread block per compute unit owns a window of
+// consecutive bags (of one sub-class, possibly spanning features).  It ranks
+// them by length in LDS, longest first, and cuts the order into rounds of gpw
+// bags; a round is pooled by one wave, one bag per lane group, so the lane
+// groups that run in lock step hold bags of nearly equal length.  Rounds are
+// dealt to the block's 16 waves in serpentine order over the four SIMDs (waves
+// w, w+4, w+8, w+12 share SIMD w & 3), which evens out the work per SIMD.  A
+// bag is still pooled whole and in id order by one lane group; there is no
+// scratch memory, atomic or pre-pass.
+constexpr int kCuThreads = 1024;
+constexpr int kCuWaves = kCuThreads / kWaveSize;
+constexpr int kMaxWindow = 2048;
+constexpr int kBagBits = 20;  // window entry = (feature index in sub-class << 20) | sample
+
+template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U>
+__global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupArgs a) {
+  constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;
+  extern __shared__ unsigned char tra_dyn_smem[];  // only its size matters (one block per CU)
+  __shared__ int64_t s_start[kMaxWindow];
+  __shared__ __align__(16) int s_len[kMaxWindow];
+  __shared__ uint32_t s_ent[kMaxWindow];
+  __shared__ uint16_t s_order[kMaxWindow];
+  __shared__ int s_rank[kMaxWindow];
+
+  TRA_STAMP(0);
+  // Block -> (sub-class, window).  Consecutive windows go to the same XCD
+  // (blocks are dealt round-robin to the 8 XCDs), so each L2 sees few tables.
+  int blk = blockIdx.x;
+  if (a.xcd_blocks > 0) blk = (blk & 7) * a.xcd_blocks + (blk >> 3);
+  int s = 0;
 #pragma unroll
-    for (int i = 0; i < NE; ++i) acc[i] *= inv;
+  for (int i = 1; i < kMaxSub; ++i)
+    if (i < a.n_sub && blk >= a.sub[i].tile_start) s = i;
+  const SubClass sc = a.sub[s];
+  const int nb_all = sc.count * a.B;
+  const int q0 = (blk - sc.tile_start) * a.window_bags;
+  if (q0 >= nb_all) return;
+  const int nb = min(a.window_bags, nb_all - q0);
+
+  for (int i = threadIdx.x; i < nb; i += kCuThreads) {
+    const int q = q0 + i;
+    const int fi = q / a.B;
+    const int b = q - fi * a.B;
+    const int64_t bag = (int64_t)a.descs[a.feats[sc.first + fi]].feature * a.B + b;
+    const int64_t st = load_index<IdxT>(a.offsets, bag);
+    s_start[i] = st;
+    s_len[i] = max(0, (int)(load_index<IdxT>(a.offsets, bag + 1) - st));
+    s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
+    s_rank[i] = 0;
   }
-  const int64_t pos = (int64_t)bag_in_feat * a.out_stride + d.out_col + (int64_t)c * NE;
-  store_outputs<NE>(a, pos, acc);
+  for (int i = nb + threadIdx.x; i < ((nb + 3) & ~3); i += kCuThreads) s_len[i] = -1;
+  __syncthreads();
+  TRA_STAMP(1);
+  // Rank sort, longest first, ties by position: a permutation of 0..nb-1.
+  // Four waves work on each bag: quarter h of the block counts the bags of
+  // quarter h of the window that rank ahead of bag i; the counts meet in LDS.
+  // Lengths are read four at a time (the tail is padded with -1).
+  {
+    const int nb4 = (nb + 3) & ~3;
+    constexpr int kQuarter = kCuThreads / 4;
+    const int h = threadIdx.x / kQuarter;
+    const int jq = ((nb4 / 4 + 3) / 4) * 4;  // int4 groups per quarter, in elements
+    const int j0 = h * jq, j1 = min(nb4, j0 + jq);
+    for (int i = threadIdx.x - h * kQuarter; i < nb4; i += kQuarter) {
+      const int li = i < nb ? s_len[i] : -1;
+      int rank = 0;
+#pragma unroll 4
+      for (int j = j0; j < j1; j += 4) {
+        const int4 l4 = *reinterpret_cast<const int4*>(&s_len[j]);
+        rank += (l4.x > li) || (l4.x == li && j < i);
+        rank += (l4.y > li) || (l4.y == li && j + 1 < i);
+        rank += (l4.z > li) || (l4.z == li && j + 2 < i);
+        rank += (l4.w > li) || (l4.w == li && j + 3 < i);
+      }
+      if (i < nb) atomicAdd(&s_rank[i], rank);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nb; i += kCuThreads) s_order[s_rank[i]] = (uint16_t)i;
+  __syncthreads();
+  TRA_STAMP(2);
+
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  const int simd = wave & 3;
+  const int lpr = sc.lpr;
+  const int gpw = kWaveSize / lpr;
+  const int g = lane / lpr;
+  const int c = lane - g * lpr;
+  const int rounds = (nb + gpw - 1) / gpw;
+  for (int slot = wave >> 2; slot * 4 < rounds; slot += kCuWaves / 4) {
+    const int r = slot * 4 + ((slot & 1) ? 3 - simd : simd);
+    if (r >= rounds) continue;
+    const int pos = r * gpw + g;
+    const bool active = g < gpw && pos < nb;
+    const int i = s_order[active ? pos : r * gpw];
+    const uint32_t ent = s_ent[i];
+    const int fi = (int)(ent >> kBagBits);
+    const int b = (int)(ent & ((1u << kBagBits) - 1));
+    const FeatureDesc d = a.descs[a.feats[sc.first + fi]];
+    const int64_t start = s_start[i];
+    const int len = active ? s_len[i] : 0;
+    const int max_len = s_len[s_order[r * gpw]];  // the round's first bag is its longest
+
+    RowWalk w;
+    w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
+    w.lane_base = a.weights + d.table_offset + w.chunk_off;
+    w.rows = d.rows;
+    w.row_bytes = d.row_bytes;
+    w.count_errors = c == 0 && d.payload_off == 0;
+
+    float acc[NE];
+#pragma unroll
+    for (int k = 0; k < NE; ++k) acc[k] = 0.0f;
+    pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+    TRA_STAMP(3);
+#ifdef TRA_INSTRUMENT
+    if (lane == 0) a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + wave) * 8 + 5] = (unsigned long long)max_len;
+#endif
+    if (active)
+      finish_bag<NE>(acc, a, len, (int64_t)b * a.out_stride + d.out_col + (int64_t)c * NE);
+    TRA_STAMP(4);
+  }
 }
 
 // ---- sequence lookup: one lane group per id, no reduction -----------------
@@ -389,13 +617,15 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
     if (i < a.n_sub && (int)blockIdx.x >= a.sub[i].tile_start) s = i;
   const int64_t stride = (int64_t)a.sub[s].tiles_per_feat * rows_per_block;
 
-  const uint8_t* table = a.weights + d.table_offset;
   const int chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
+  const uint8_t* lane_base = a.weights + d.table_offset + chunk_off;
   const bool count_errors = c == 0 && d.payload_off == 0;
   for (int64_t j = first + (int64_t)tile * rows_per_block + wave * gpw + g; j < last;
        j += stride) {
     RowBuf<CB> r;
-    fetch_row<DTYPE, CB, IdxT, false>(r, true, j, a, table, d.rows, d.row_bytes, chunk_off, count_errors);
+    const int bad = fetch_row<DTYPE, CB, false>(r, load_index<IdxT>(a.indices, j), j, a, lane_base,
+                                                 d.rows, d.row_bytes, chunk_off);
+    if (bad && count_errors) atomicAdd(a.err_count, 1ull);
     float acc[NE];
 #pragma unroll
     for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
@@ -414,47 +644,65 @@ struct LaunchClass {
   int32_t* feats_dev = nullptr;
 };
 
+struct LaunchParams {
+  int grid;
+  int balanced;   // 1: one 1024-thread block per window of bags (tbe_pooled_cu_kernel)
+  int lds_bytes;  // dynamic LDS of the balanced kernel (sized so one block fits per CU)
+  int unroll;     // rows per pipeline batch: 2, 4 or 8
+  bool idx64;
+  bool weighted;
+  bool nobag;
+};
+
 template <int DTYPE>
-int launch_lookup(const LaunchClass& cls, LookupArgs a, int cb, bool idx64, bool weighted,
-                  bool nobag, int grid, hipStream_t stream);
+int launch_lookup(const LookupArgs& a, int cb, const LaunchParams& p, hipStream_t stream);
+
+template <int DTYPE, int CB, typename IdxT>
+void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream) {
+  dim3 g(p.grid);
+  if (p.nobag) {
+    hipLaunchKernelGGL((tbe_nobag_kernel<DTYPE, CB, IdxT>), g, dim3(kBlockThreads), 0, stream, a);
+    return;
+  }
+#define TRA_POOLED(W, U)                                                                       \
+  do {                                                                                         \
+    if (p.balanced)                                                                            \
+      hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kCuThreads),   \
+                         p.lds_bytes, stream, a);                                              \
+    else                                                                                       \
+      hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kBlockThreads), 0, \
+                         stream, a);                                                           \
+  } while (0)
+  if (p.weighted) {
+    if (p.unroll >= 8) TRA_POOLED(true, 8); else if (p.unroll >= 4) TRA_POOLED(true, 4); else TRA_POOLED(true, 2);
+  } else {
+    if (p.unroll >= 8) TRA_POOLED(false, 8); else if (p.unroll >= 4) TRA_POOLED(false, 4); else TRA_POOLED(false, 2);
+  }
+#undef TRA_POOLED
+}
 
 template <int DTYPE, int CB>
-int launch_lookup_cb(LookupArgs a, bool idx64, bool weighted, bool nobag, int grid,
-                     hipStream_t stream) {
-  constexpr int U = 4;
-  dim3 g(grid), b(kBlockThreads);
-  if (nobag) {
-    if (idx64)
-      hipLaunchKernelGGL((tbe_nobag_kernel<DTYPE, CB, int64_t>), g, b, 0, stream, a);
-    else
-      hipLaunchKernelGGL((tbe_nobag_kernel<DTYPE, CB, int32_t>), g, b, 0, stream, a);
-  } else if (weighted) {
-    if (idx64)
-      hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, int64_t, true, U>), g, b, 0, stream, a);
-    else
-      hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, int32_t, true, U>), g, b, 0, stream, a);
-  } else {
-    if (idx64)
-      hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, int64_t, false, U>), g, b, 0, stream, a);
-    else
-      hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, int32_t, false, U>), g, b, 0, stream, a);
-  }
+int launch_lookup_cb(const LookupArgs& a, const LaunchParams& p, hipStream_t stream) {
+  if (p.idx64)
+    launch_typed<DTYPE, CB, int64_t>(a, p, stream);
+  else
+    launch_typed<DTYPE, CB, int32_t>(a, p, stream);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, "tbe lookup launch");
   return TRA_OK;
 }
 
-#define TRA_DEFINE_LAUNCH(DTYPE)                                                        \
-  template <>                                                                           \
-  int launch_lookup<DTYPE>(const LaunchClass&, LookupArgs a, int cb, bool idx64,        \
-                           bool weighted, bool nobag, int grid, hipStream_t stream) {   \
-    switch (cb) {                                                                       \
-      case 16: return launch_lookup_cb<DTYPE, 16>(a, idx64, weighted, nobag, grid, stream); \
-      case 8: return launch_lookup_cb<DTYPE, 8>(a, idx64, weighted, nobag, grid, stream);   \
-      case 4: return launch_lookup_cb<DTYPE, 4>(a, idx64, weighted, nobag, grid, stream);   \
-    }                                                                                   \
-    set_error("bad chunk size %d", cb);                                                 \
-    return TRA_ERR_INVALID_ARGUMENT;                                                    \
+#define TRA_DEFINE_LAUNCH(DTYPE)                                                          \
+  template <>                                                                             \
+  int launch_lookup<DTYPE>(const LookupArgs& a, int cb, const LaunchParams& p,            \
+                           hipStream_t stream) {                                          \
+    switch (cb) {                                                                         \
+      case 16: return launch_lookup_cb<DTYPE, 16>(a, p, stream);                          \
+      case 8: return launch_lookup_cb<DTYPE, 8>(a, p, stream);                            \
+      case 4: return launch_lookup_cb<DTYPE, 4>(a, p, stream);                            \
+    }                                                                                     \
+    set_error("bad chunk size %d", cb);                                                   \
+    return TRA_ERR_INVALID_ARGUMENT;                                                      \
   }
 
 }  // namespace tra

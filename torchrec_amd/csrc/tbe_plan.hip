@@ -1,6 +1,7 @@
 // Host side of the TBE lookup: plan construction (tra_tbe_create) and launch
 // (tra_tbe_forward), plus the small library-level entry points.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <string>
@@ -25,15 +26,48 @@ int hip_fail(hipError_t e, const char* what) {
 
 // Explicit specializations live in tbe_lookup_<dtype>.hip.
 template <>
-int launch_lookup<TRA_INT8>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+int launch_lookup<TRA_INT8>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
-int launch_lookup<TRA_INT4>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+int launch_lookup<TRA_INT4>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
-int launch_lookup<TRA_INT2>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+int launch_lookup<TRA_INT2>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
-int launch_lookup<TRA_FP16>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+int launch_lookup<TRA_FP16>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
-int launch_lookup<TRA_FP32>(const LaunchClass&, LookupArgs, int, bool, bool, bool, int, hipStream_t);
+int launch_lookup<TRA_FP32>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
+
+// Launch shape of the pooled kernels.  Defaults are chosen per call from the
+// problem size; TRA_BALANCED / TRA_WINDOW / TRA_UNROLL / TRA_LDS override them
+// (tuning).
+struct Tuning {
+  int balanced;  // 1: tbe_pooled_cu_kernel, one block per CU-sized window of bags
+  int window;    // bags per block (0: derive from the problem size)
+  int unroll;
+  int lds_bytes;
+};
+
+static int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : fallback;
+}
+
+constexpr int kNumCus = 256;
+
+static Tuning choose_tuning(int64_t bags, int64_t num_indices) {
+  Tuning t;
+  // Ranking bags by length pays once every CU has several rounds to balance.
+  t.balanced = bags >= 128 * kNumCus && num_indices >= 2048 * (int64_t)kNumCus;
+  t.window = 0;
+  t.unroll = 4;
+  t.lds_bytes = 48 * 1024;  // with the static arrays > half of a CU's LDS: one block per CU
+  t.balanced = env_int("TRA_BALANCED", t.balanced);
+  t.window = env_int("TRA_WINDOW", t.window);
+  t.unroll = env_int("TRA_UNROLL", t.unroll);
+  t.lds_bytes = env_int("TRA_LDS", t.lds_bytes);
+  if (t.window > kMaxWindow) t.window = kMaxWindow;
+  if (t.window < 0) t.window = 0;
+  return t;
+}
 
 }  // namespace tra
 
@@ -94,7 +128,12 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
       set_error("table %d: unsupported dtype %d", t, s.dtype);
       return TRA_ERR_INVALID_ARGUMENT;
     }
-    if (s.dim <= 0 || s.rows < 0 || (int64_t)s.dim * bits % 32 != 0) {
+    if (s.rows < 1) {
+      // Skipped ids are redirected to row 0, so every table needs one.
+      set_error("table %d has no rows", t);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+    if (s.dim <= 0 || (int64_t)s.dim * bits % 32 != 0) {
       set_error("table %d: dim %d with %d-bit elements is not a whole number of dwords", t,
                 s.dim, bits);
       return TRA_ERR_INVALID_ARGUMENT;
@@ -124,7 +163,11 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     if (s.dim != plan->dim0) plan->same_dim = false;
     const int bits = bits_of(s.dtype);
     const int payload = s.dim * bits / 8;
-    const int cb = payload % 16 == 0 ? 16 : (payload % 8 == 0 ? 8 : 4);
+    int cb = payload % 16 == 0 ? 16 : (payload % 8 == 0 ? 8 : 4);
+    {
+      const int force = env_int("TRA_CB", 0);  // tuning: smaller lane chunks
+      if ((force == 8 || force == 4) && force < cb && payload % force == 0) cb = force;
+    }
     const int max_slice = cb * kWaveSize;  // bytes one wave-wide lane group covers
     for (int off = 0; off < payload; off += max_slice) {
       const int bytes = std::min(max_slice, payload - off);
@@ -232,6 +275,10 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
   }
   const bool nobag = pooling_mode == TRA_POOL_NONE;
   if (tbe->num_features == 0 || batch_size == 0 || (nobag && num_indices == 0)) return TRA_OK;
+  if (num_indices < 0) {
+    set_error("tra_tbe_forward: num_indices is required");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
   if (!weights || !offsets || !out || (!indices && num_indices != 0)) {
     set_error("tra_tbe_forward: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
@@ -242,19 +289,27 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
   }
   const int esz = out_dtype == TRA_FP16 ? 2 : 4;
   hipStream_t s = (hipStream_t)stream;
+  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
+  bool balanced = !nobag && tune.balanced && batch_size <= (1 << kBagBits);
+  for (const LaunchClass& cls : tbe->classes)
+    if ((int64_t)cls.feats.size() >= (int64_t(1) << (32 - kBagBits)) ||
+        (int64_t)cls.feats.size() * batch_size >= (int64_t(1) << 31))
+      balanced = false;
   for (const LaunchClass& cls : tbe->classes) {
     LookupArgs a;
     memset(&a, 0, sizeof(a));
     a.weights = (const uint8_t*)weights;
     a.descs = tbe->slices_dev;
     a.feats = cls.feats_dev;
-    a.indices = indices;
+    // Lanes past the end of their bag still issue (clamped) id loads, so the
+    // kernels need one readable element even when there are no ids at all.
+    a.indices = num_indices > 0 ? indices : (const void*)tbe->err_dev;
     a.offsets = offsets;
     a.psw = nobag ? nullptr : per_sample_weights;
     a.out = out;
     a.out_stride = out_stride;
     a.err_count = tbe->err_dev;
-    a.num_indices = num_indices;
+    a.num_indices = num_indices > 0 ? num_indices : 1;
     a.B = batch_size;
     a.mean = pooling_mode == TRA_POOL_MEAN;
     a.out_fp16 = out_dtype == TRA_FP16;
@@ -268,6 +323,19 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
     if (!nobag)
       for (int id : cls.feats) vec = vec && ((int64_t)tbe->slices[id].out_col * esz % 16 == 0);
     a.vec_store = vec;
+    int window = 0;
+    if (balanced) {
+      // One window per CU when that fits the LDS arrays, else several per CU.
+      window = tune.window;
+      if (window == 0) {
+        const int64_t class_bags = (int64_t)cls.feats.size() * batch_size;
+        const int64_t per_cu = (class_bags + kNumCus - 1) / kNumCus;
+        const int64_t passes = (per_cu + kMaxWindow - 1) / kMaxWindow;
+        window = (int)((per_cu + passes - 1) / passes);
+        if (window < 64) window = 64;
+      }
+      a.window_bags = window;
+    }
     int grid = 0;
     int n_sub = 0;
     for (size_t i = 0; i < cls.feats.size();) {
@@ -277,30 +345,47 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
       sc.first = (int)i;
       sc.count = (int)(j - i);
       sc.lpr = cls.lprs[i];
-      const int per_block = kWavesPerBlock * (kWaveSize / sc.lpr);
+      const int gpw = kWaveSize / sc.lpr;
+      const int per_block = kWavesPerBlock * gpw;
+      sc.tile_start = grid;
       if (nobag) {
         // Blocks stride over a feature's ids; enough blocks for ~the average
         // feature, capped so the grid stays modest.
         int64_t avg = num_indices > 0 ? num_indices / tbe->num_features + 1 : 4096;
         int64_t t = (avg + per_block - 1) / per_block;
         sc.tiles_per_feat = (int)std::max<int64_t>(1, std::min<int64_t>(t, 8192));
+        grid += sc.count * sc.tiles_per_feat;
+      } else if (balanced) {
+        const int64_t nb = (int64_t)sc.count * batch_size;
+        sc.tiles_per_feat = 0;
+        grid += (int)((nb + window - 1) / window);
       } else {
         sc.tiles_per_feat = (batch_size + per_block - 1) / per_block;
+        grid += sc.count * sc.tiles_per_feat;
       }
-      sc.tile_start = grid;
-      grid += sc.count * sc.tiles_per_feat;
       i = j;
     }
     a.n_sub = n_sub;
+    LaunchParams lp;
+    lp.balanced = balanced ? 1 : 0;
+    lp.lds_bytes = tune.lds_bytes;
+    lp.grid = grid;
+    if (balanced) {
+      // XCD remap needs a grid that is a multiple of 8 (surplus blocks exit at once).
+      lp.grid = (grid + 7) / 8 * 8;
+      a.xcd_blocks = env_int("TRA_XCD", 1) ? lp.grid / 8 : 0;
+    }
+    lp.unroll = tune.unroll;
+    lp.idx64 = idx_is_i64 != 0;
+    lp.weighted = a.psw != nullptr;
+    lp.nobag = nobag;
     int rc;
-    const bool i64 = idx_is_i64 != 0;
-    const bool w = a.psw != nullptr;
     switch (cls.dtype) {
-      case TRA_INT8: rc = launch_lookup<TRA_INT8>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
-      case TRA_INT4: rc = launch_lookup<TRA_INT4>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
-      case TRA_INT2: rc = launch_lookup<TRA_INT2>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
-      case TRA_FP16: rc = launch_lookup<TRA_FP16>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
-      default: rc = launch_lookup<TRA_FP32>(cls, a, cls.cb, i64, w, nobag, grid, s); break;
+      case TRA_INT8: rc = launch_lookup<TRA_INT8>(a, cls.cb, lp, s); break;
+      case TRA_INT4: rc = launch_lookup<TRA_INT4>(a, cls.cb, lp, s); break;
+      case TRA_INT2: rc = launch_lookup<TRA_INT2>(a, cls.cb, lp, s); break;
+      case TRA_FP16: rc = launch_lookup<TRA_FP16>(a, cls.cb, lp, s); break;
+      default: rc = launch_lookup<TRA_FP32>(a, cls.cb, lp, s); break;
     }
     if (rc != TRA_OK) return rc;
   }
