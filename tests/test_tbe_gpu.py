@@ -196,3 +196,159 @@ def test_properties_large():
     order = list(rng.permutation(T))
     p = mk(PoolingMode.SUM, order)(ti, to, feature_positions=order, batch_size=B)
     assert torch.equal(p.view(B, T, dim), a.view(B, T, dim)[:, order, :])
+
+
+# The pooled lookup has two kernels: a static bag->wave mapping for small calls
+# and a per-CU window kernel that ranks bags by length (taken when a call has
+# at least 32768 bags and 524288 ids).  TRA_BALANCED / TRA_WINDOW are the
+# library's tuning overrides; the tests below use them to put oracle-sized
+# inputs through the window kernel.
+
+@pytest.mark.parametrize("dtype", [O.INT8, O.INT4, O.INT2, O.FP16, O.FP32])
+@pytest.mark.parametrize("pooling,weighted", [(O.SUM, False), (O.SUM, True), (O.MEAN, False), (O.MEAN, True)])
+def test_window_kernel_bit_exact(monkeypatch, dtype, pooling, weighted):
+    """Window kernel vs oracle: every weight type x pooling, both id widths and
+    output types, several windows per feature and a ragged last window."""
+    monkeypatch.setenv("TRA_BALANCED", "1")
+    rng = np.random.default_rng(900 + dtype * 10 + pooling + weighted)
+    for dim, out_dtype, idt, window in ((128, O.FP32, np.int32, 64), (64, O.FP16, np.int64, 100),
+                                        (256, O.FP16, np.int32, 0), (32, O.FP32, np.int64, 2048)):
+        monkeypatch.setenv("TRA_WINDOW", str(window))
+        rows, B = 3000, 211
+        specs = [(dtype, rows, dim), (dtype, rows + 13, dim)]
+        ftm = [0, 1, 0]
+        tbe, store = build(rng, specs, ftm, pooling, out_dtype, 16)
+        lengths, offsets, ids = make_bags(rng, [rows, rows + 13, rows], B, 60, idt)
+        psw = rng.uniform(-1, 1, len(ids)).astype(np.float32) if weighted else None
+        got, want = run_both(tbe, store, ftm, B, ids, offsets, psw, pooling, out_dtype)
+        assert bits_equal(got, want) == 0, (dim, out_dtype, idt, window)
+        assert tbe.out_of_range_count() == 0
+
+
+def test_window_kernel_mixed_and_edges(monkeypatch):
+    """Window kernel: one group mixing weight types and dims (several launch
+    classes and sub-classes), bags longer than the exact length bins, empty
+    bags, -1 and out-of-range ids, and a key order that differs from the
+    operator's feature order."""
+    monkeypatch.setenv("TRA_BALANCED", "1")
+    monkeypatch.setenv("TRA_WINDOW", "96")
+    rng = np.random.default_rng(41)
+    specs = [([O.INT8, O.INT4, O.INT2, O.FP16][(t // 4) % 4], 500 + 7 * t, [32, 64, 128, 256][t % 4]) for t in range(16)]
+    ftm = list(range(16))
+    tbe, store = build(rng, specs, ftm, O.SUM, O.FP32, 16)
+    B = 77
+    lengths, offsets, ids = make_bags(rng, [s[1] for s in specs], B, 40)
+    psw = rng.uniform(0, 1, len(ids)).astype(np.float32)
+    got, want = run_both(tbe, store, ftm, B, ids, offsets, psw, O.SUM, O.FP32)
+    assert bits_equal(got, want) == 0
+
+    rows, dim, B = 1000, 128, 40
+    tbe, store = build(rng, [(O.INT4, rows, dim)], [0, 0], O.MEAN, O.FP16, 16)
+    lens = rng.integers(0, 30, 2 * B)
+    lens[3], lens[50], lens[51] = 700, 5000, 193   # coarse bins, last bin, first coarse bin
+    lens[10:20] = 0
+    offsets = np.zeros(2 * B + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(lens)
+    ids = rng.integers(0, rows, offsets[-1]).astype(np.int32)
+    ids[::7] = -1
+    got, want = run_both(tbe, store, [0, 0], B, ids, offsets, None, O.MEAN, O.FP16)
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
+    bad = ids.copy()
+    pos = np.flatnonzero(bad >= 0)[:9]
+    bad[pos] = rows + 5
+    got = tbe(torch.from_numpy(bad).to(DEV), torch.from_numpy(offsets).to(DEV)).cpu().numpy()
+    bad[pos] = -1
+    want = O.tbe_forward(store, [0, 0], B, bad, offsets, None, O.MEAN, O.FP16)
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 9
+
+    # all bags empty
+    z = np.zeros(2 * B + 1, dtype=np.int32)
+    got, want = run_both(tbe, store, [0, 0], B, np.zeros(0, dtype=np.int32), z, None, O.MEAN, O.FP16)
+    assert bits_equal(got, want) == 0 and not got.any()
+
+    # keys [f1, unused, f0] read in place, written into a slice of a wider output
+    rows, dim, B = 800, 64, 133
+    tbe, store = build(rng, [(O.INT8, rows, dim), (O.INT4, rows, dim)], [0, 1], O.SUM, O.FP32, 16)
+    lengths, offsets, ids = make_bags(rng, [rows, rows, rows], B, 20)
+    out = torch.full((B, 3 * dim + 5), 7.0, device=DEV)
+    tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV), feature_positions=[2, 0],
+        batch_size=B, out=out, out_col=dim)
+    seg = [ids[offsets[k * B]:offsets[(k + 1) * B]] for k in range(3)]
+    L = lengths.reshape(3, B)
+    o_off = np.zeros(2 * B + 1, dtype=np.int32)
+    o_off[1:] = np.cumsum(np.concatenate([L[2], L[0]]))
+    want = O.tbe_forward(store, [0, 1], B, np.concatenate([seg[2], seg[0]]), o_off, None, O.SUM, O.FP32)
+    got = out.cpu().numpy()
+    assert bits_equal(np.ascontiguousarray(got[:, dim:3 * dim]), want) == 0
+    assert (got[:, :dim] == 7.0).all() and (got[:, 3 * dim:] == 7.0).all()
+
+
+def test_window_kernel_equals_static_at_scale(monkeypatch):
+    """At a size where the window kernel is the default (26 features x 2048
+    samples, ~1M ids) both kernels give the same bits, and a sample of bags
+    matches the oracle."""
+    rng = np.random.default_rng(2024)
+    T, rows, dim, B = 26, 50_000, 128, 2048
+    specs = [(O.INT4, rows, dim)] * T
+    ftm = list(range(T))
+    tbe, store = build(rng, specs, ftm, O.SUM, O.FP16, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 40, empty_frac=0.02)
+    ti, to = torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV)
+    monkeypatch.delenv("TRA_BALANCED", raising=False)
+    monkeypatch.delenv("TRA_WINDOW", raising=False)
+    a = tbe(ti, to)
+    monkeypatch.setenv("TRA_BALANCED", "0")
+    b = tbe(ti, to)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    # oracle on the first 64 samples of every feature
+    Bs = 64
+    sub_len = lengths.reshape(T, B)[:, :Bs]
+    sub_off = np.zeros(T * Bs + 1, dtype=np.int32)
+    sub_off[1:] = np.cumsum(sub_len.reshape(-1))
+    sub_ids = np.concatenate([ids[offsets[f * B]:offsets[f * B + Bs]] for f in range(T)])
+    want = O.tbe_forward(store, ftm, Bs, sub_ids, sub_off, None, O.SUM, O.FP16)
+    assert bits_equal(np.ascontiguousarray(a[:Bs].cpu().numpy()), want) == 0
+
+
+def test_lookup_under_hip_graph():
+    """The lookup captured in a HIP graph: several replays, with eager work and
+    synchronisation in between, each equal to the eager result."""
+    rng = np.random.default_rng(8)
+    T, rows, dim, B = 6, 5000, 128, 256
+    specs = [(O.INT4, rows, dim)] * T
+    tbe, store = build(rng, specs, list(range(T)), O.SUM, O.FP16, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 30)
+    cap = int(len(ids) * 1.5)
+    ti = torch.zeros(cap, dtype=torch.int32, device=DEV)
+    to = torch.zeros(T * B + 1, dtype=torch.int32, device=DEV)
+    out = torch.zeros(B, T * dim, dtype=torch.float16, device=DEV)
+
+    def load(seed):
+        r = np.random.default_rng(seed)
+        l, o, i = make_bags(r, [rows] * T, B, 30)
+        assert len(i) <= cap
+        ti.zero_()
+        ti[: len(i)].copy_(torch.from_numpy(i))
+        to.copy_(torch.from_numpy(o))
+        return i, o
+
+    load(0)
+    tbe(ti, to, batch_size=B, out=out)  # plan creation outside capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            tbe(ti, to, batch_size=B, out=out)
+    torch.cuda.synchronize()
+    for seed in (1, 2, 3, 4):
+        i, o = load(seed)
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().copy()
+        eager = tbe(ti, to, batch_size=B).cpu().numpy()
+        want = O.tbe_forward(store, list(range(T)), B, i, o, None, O.SUM, O.FP16)
+        assert bits_equal(got, want) == 0, seed
+        assert bits_equal(eager, want) == 0, seed

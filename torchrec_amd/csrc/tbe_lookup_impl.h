@@ -24,6 +24,7 @@ namespace tra {
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlockThreads = kWavesPerBlock * kWaveSize;
 constexpr int kMaxSub = 8;
+constexpr int kMaxPos = 128;
 
 // Features of one launch that share LPR (i.e. share dim).
 struct SubClass {
@@ -52,6 +53,7 @@ struct LookupArgs {
   int32_t out_fp16;
   int32_t window_bags;  // balanced pooled kernel: bags per block
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
+  int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
 #ifdef TRA_INSTRUMENT
   unsigned long long* ts;  // [waves][8] wall-clock stamps
 #endif
@@ -480,6 +482,13 @@ constexpr int kCuWaves = kCuThreads / kWaveSize;
 constexpr int kMaxWindow = 2048;
 constexpr int kBagBits = 20;  // window entry = (feature index in sub-class << 20) | sample
 
+constexpr int kLenBins = 256;
+
+// Sort key of a bag length: exact below 192, then steps of 64, then one bin.
+__device__ __forceinline__ int length_bin(int len) {
+  return len < 192 ? len : min(kLenBins - 1, 192 + ((len - 192) >> 6));
+}
+
 template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U>
 __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;
@@ -488,7 +497,8 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   __shared__ __align__(16) int s_len[kMaxWindow];
   __shared__ uint32_t s_ent[kMaxWindow];
   __shared__ uint16_t s_order[kMaxWindow];
-  __shared__ int s_rank[kMaxWindow];
+  __shared__ uint16_t s_slot[kMaxWindow];
+  __shared__ int s_hist[kLenBins];
 
   TRA_STAMP(0);
   // Block -> (sub-class, window).  Consecutive windows go to the same XCD
@@ -505,46 +515,54 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   if (q0 >= nb_all) return;
   const int nb = min(a.window_bags, nb_all - q0);
 
+  if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
+  __syncthreads();
   for (int i = threadIdx.x; i < nb; i += kCuThreads) {
     const int q = q0 + i;
     const int fi = q / a.B;
     const int b = q - fi * a.B;
-    const int64_t bag = (int64_t)a.descs[a.feats[sc.first + fi]].feature * a.B + b;
+    // Position of the bag's feature among the input keys: from the launch
+    // arguments when the class is small enough, else from the descriptors.
+    const int fpos = sc.first + fi < kMaxPos ? (int)a.feat_pos[sc.first + fi]
+                                             : a.descs[a.feats[sc.first + fi]].feature;
+    const int64_t bag = (int64_t)fpos * a.B + b;
     const int64_t st = load_index<IdxT>(a.offsets, bag);
     s_start[i] = st;
-    s_len[i] = max(0, (int)(load_index<IdxT>(a.offsets, bag + 1) - st));
+    const int len = max(0, (int)(load_index<IdxT>(a.offsets, bag + 1) - st));
+    s_len[i] = len;
     s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
-    s_rank[i] = 0;
+    s_slot[i] = (uint16_t)atomicAdd(&s_hist[length_bin(len)], 1);
   }
-  for (int i = nb + threadIdx.x; i < ((nb + 3) & ~3); i += kCuThreads) s_len[i] = -1;
   __syncthreads();
   TRA_STAMP(1);
-  // Rank sort, longest first, ties by position: a permutation of 0..nb-1.
-  // Four waves work on each bag: quarter h of the block counts the bags of
-  // quarter h of the window that rank ahead of bag i; the counts meet in LDS.
-  // Lengths are read four at a time (the tail is padded with -1).
-  {
-    const int nb4 = (nb + 3) & ~3;
-    constexpr int kQuarter = kCuThreads / 4;
-    const int h = threadIdx.x / kQuarter;
-    const int jq = ((nb4 / 4 + 3) / 4) * 4;  // int4 groups per quarter, in elements
-    const int j0 = h * jq, j1 = min(nb4, j0 + jq);
-    for (int i = threadIdx.x - h * kQuarter; i < nb4; i += kQuarter) {
-      const int li = i < nb ? s_len[i] : -1;
-      int rank = 0;
-#pragma unroll 4
-      for (int j = j0; j < j1; j += 4) {
-        const int4 l4 = *reinterpret_cast<const int4*>(&s_len[j]);
-        rank += (l4.x > li) || (l4.x == li && j < i);
-        rank += (l4.y > li) || (l4.y == li && j + 1 < i);
-        rank += (l4.z > li) || (l4.z == li && j + 2 < i);
-        rank += (l4.w > li) || (l4.w == li && j + 3 < i);
-      }
-      if (i < nb) atomicAdd(&s_rank[i], rank);
+  // Counting sort, longest first: a permutation of 0..nb-1.  hist[] holds the
+  // bin sizes and every bag already has its slot within its bin; one wave
+  // turns the sizes into start positions (bins in descending order).
+  if (threadIdx.x < kWaveSize) {
+    const int l = threadIdx.x;
+    int h[kLenBins / kWaveSize];
+    int sum = 0;
+#pragma unroll
+    for (int k = 0; k < kLenBins / kWaveSize; ++k) {
+      h[k] = s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)];
+      sum += h[k];
+    }
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < kWaveSize; d <<= 1) {
+      const int up = __shfl_up(incl, d, kWaveSize);
+      if (l >= d) incl += up;
+    }
+    int base = incl - sum;
+#pragma unroll
+    for (int k = 0; k < kLenBins / kWaveSize; ++k) {
+      s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)] = base;
+      base += h[k];
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += kCuThreads) s_order[s_rank[i]] = (uint16_t)i;
+  for (int i = threadIdx.x; i < nb; i += kCuThreads)
+    s_order[s_hist[length_bin(s_len[i])] + s_slot[i]] = (uint16_t)i;
   __syncthreads();
   TRA_STAMP(2);
 

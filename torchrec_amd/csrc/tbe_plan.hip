@@ -163,7 +163,9 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     if (s.dim != plan->dim0) plan->same_dim = false;
     const int bits = bits_of(s.dtype);
     const int payload = s.dim * bits / 8;
-    int cb = payload % 16 == 0 ? 16 : (payload % 8 == 0 ? 8 : 4);
+    // Bytes per lane.  Rows of up to 64 payload bytes take 8-byte chunks: more
+    // lanes per row means fewer bags per wave, which balances better.
+    int cb = payload % 16 == 0 && payload > 64 ? 16 : (payload % 8 == 0 ? 8 : 4);
     {
       const int force = env_int("TRA_CB", 0);  // tuning: smaller lane chunks
       if ((force == 8 || force == 4) && force < cb && payload % force == 0) cb = force;
@@ -291,6 +293,8 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
   hipStream_t s = (hipStream_t)stream;
   const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
   bool balanced = !nobag && tune.balanced && batch_size <= (1 << kBagBits);
+  for (const FeatureDesc& d : tbe->slices)
+    if (d.feature > 32767) balanced = false;
   for (const LaunchClass& cls : tbe->classes)
     if ((int64_t)cls.feats.size() >= (int64_t(1) << (32 - kBagBits)) ||
         (int64_t)cls.feats.size() * batch_size >= (int64_t(1) << 31))
@@ -335,6 +339,8 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
         if (window < 64) window = 64;
       }
       a.window_bags = window;
+      for (size_t i = 0; i < cls.feats.size() && i < (size_t)kMaxPos; ++i)
+        a.feat_pos[i] = (int16_t)tbe->slices[cls.feats[i]].feature;
     }
     int grid = 0;
     int n_sub = 0;
