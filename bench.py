@@ -9,9 +9,10 @@ Zipf(1.05) over a seeded permutation of each table's rows.  Synthetic, seeded.
 
 A step is one QuantEmbeddingBagCollection.forward over one KeyedJaggedTensor
 (lengths -> offsets scan + the pooled lookup), inputs resident in HBM; steps
-rotate over --batches distinct id batches.  By default each batch's forward is
-captured once in a HIP graph and the timed loop replays the graphs
-(--mode eager times the plain Python calls instead; both are reported).
+rotate over --batches distinct id batches.  The timed loop makes the plain
+Python calls (--mode graph captures each batch's forward in a HIP graph and
+replays the graphs instead; on this stack a graph launch costs more than the
+two kernel launches it replaces, so it is not the default).
 
 One JSON line is printed: the metric (pooled lookups/s), the roofline of the
 lookup kernel (algorithmic bytes / HIP-event duration against 8 TB/s) and the
@@ -20,6 +21,7 @@ CPU baseline (fbgemm's own kernels on the host cores, bounded sample).
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import math
 import os
@@ -31,6 +33,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+CAL_COPY_BYTES = 1 << 28
 
 
 def parse_args():
@@ -40,10 +43,13 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=200)
     p.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     p.add_argument("--batches", type=int, default=8, help="distinct id batches rotated through")
-    p.add_argument("--mode", default="graph", choices=["graph", "eager"])
+    p.add_argument("--mode", default="eager", choices=["graph", "eager"])
     p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline sample")
+    p.add_argument("--rocprof-summary", metavar="DIR", default=None,
+                   help="no benchmark: summarize rocprofv3 CSV output under DIR (kernel_stats / counter_collection) "
+                        "for this library's kernels and exit")
     p.add_argument("--scale", type=float, default=1.0, help="shrink table rows (debug only; result is then invalid)")
     return p.parse_args()
 
@@ -223,6 +229,9 @@ def build_workload(args, dev):
 # CPU baseline (fbgemm kernels from libtorch_cpu on the host cores)
 # --------------------------------------------------------------------------
 def cpu_baseline(wl, out_gpu, seconds):
+    """fbgemm's CPU kernels (the ones the reference's CPU path runs) over the same
+    batches, bags split over the host threads.  The whole packed store is copied
+    to host memory when it fits; otherwise only the rows the batches touch."""
     import numpy as np
     import torch
 
@@ -231,69 +240,115 @@ def cpu_baseline(wl, out_gpu, seconds):
     module = wl["module"]
     tbe = module._emb_modules[0]
     code = {"fp32": O.FP32, "fp16": O.FP16, "int8": O.INT8, "int4": O.INT4, "int2": O.INT2}
-    values, lengths, w = wl["batches"][0]
     T, B = wl["T"], wl["B"]
-    ids = values.cpu().numpy()
-    offs = np.zeros(T * B + 1, dtype=np.int32)
-    offs[1:] = np.cumsum(lengths.cpu().numpy())
-    # compact the touched rows so the host never needs the whole store
-    comp_tables, new_ids, pos = [], np.empty_like(ids), 0
-    offsets_t, rows_t, base = [], [], 0
-    pieces = []
-    for t in range(T):
-        seg = ids[offs[t * B]: offs[(t + 1) * B]]
-        uniq, inv = np.unique(seg, return_inverse=True)
-        new_ids[pos:pos + len(seg)] = inv
-        pos += len(seg)
-        rb = tbe.row_bytes[t]
-        view = tbe._rows_view(t)
-        rows = view[torch.from_numpy(uniq.astype(np.int64)).to(view.device)].cpu().numpy() if len(uniq) else np.zeros((0, rb), np.uint8)
-        pieces.append(rows.reshape(-1))
-        offsets_t.append(base)
-        rows_t.append(len(uniq))
-        base += O.round_up(rows.size, 128)
-        pieces.append(np.zeros(base - offsets_t[-1] - rows.size, dtype=np.uint8))
-    store = O.Store(
-        np.concatenate(pieces) if pieces else np.zeros(1, np.uint8),
-        np.asarray(offsets_t, dtype=np.int64), np.asarray(rows_t, dtype=np.int64),
-        np.asarray(tbe.dims, dtype=np.int32), np.asarray([code[str(x)] for x in tbe.weight_tys], dtype=np.int32),
-        np.asarray(tbe.row_bytes, dtype=np.int32),
-    )
-    psw = None if w is None else w.cpu().numpy()
+    NB = len(wl["batches"])
+    host = []
+    for values, lengths, w in wl["batches"]:
+        offs = np.zeros(T * B + 1, dtype=np.int32)
+        offs[1:] = np.cumsum(lengths.cpu().numpy())
+        host.append([values.cpu().numpy(), offs, None if w is None else w.cpu().numpy()])
+    try:
+        avail = os.sysconf("SC_AVPHYS_PAGES") * os.sysconf("SC_PAGE_SIZE")
+    except (ValueError, OSError):
+        avail = 0
+    whole = tbe.weights_size * 1.3 < avail and tbe.weights_size < 64e9
+    if whole:
+        store = O.Store(
+            tbe.weights_dev.cpu().numpy(),
+            np.asarray(tbe.weights_physical_offsets, dtype=np.int64), np.asarray(tbe.rows, dtype=np.int64),
+            np.asarray(tbe.dims, dtype=np.int32), np.asarray([code[str(x)] for x in tbe.weight_tys], dtype=np.int32),
+            np.asarray(tbe.row_bytes, dtype=np.int32),
+        )
+        where = f"whole {tbe.weights_size / 1e9:.2f} GB store in host memory"
+    else:
+        # compact the rows any batch touches (the store does not fit the host)
+        pieces, offsets_t, rows_t, base = [], [], [], 0
+        for t in range(T):
+            segs = [h[0][h[1][t * B]: h[1][(t + 1) * B]] for h in host]
+            uniq = np.unique(np.concatenate(segs))
+            for h in host:
+                lo, hi = h[1][t * B], h[1][(t + 1) * B]
+                h[0][lo:hi] = np.searchsorted(uniq, h[0][lo:hi])
+            rb = tbe.row_bytes[t]
+            view = tbe._rows_view(t)
+            rows = view[torch.from_numpy(uniq.astype(np.int64)).to(view.device)].cpu().numpy() if len(uniq) else np.zeros((0, rb), np.uint8)
+            pieces.append(rows.reshape(-1))
+            offsets_t.append(base)
+            rows_t.append(len(uniq))
+            base += O.round_up(rows.size, 128)
+            pieces.append(np.zeros(base - offsets_t[-1] - rows.size, dtype=np.uint8))
+        store = O.Store(
+            np.concatenate(pieces), np.asarray(offsets_t, dtype=np.int64), np.asarray(rows_t, dtype=np.int64),
+            np.asarray(tbe.dims, dtype=np.int32), np.asarray([code[str(x)] for x in tbe.weight_tys], dtype=np.int32),
+            np.asarray(tbe.row_bytes, dtype=np.int32),
+        )
+        where = (f"store too large for the host: tables compacted to the {int(sum(rows_t))} rows the batches touch "
+                 f"({base / 1e9:.2f} GB), which flatters the CPU's cache hit rate")
     pooling = int(tbe.pooling_mode)
     odt = O.FP16 if wl["out_dtype"] == torch.half else O.FP32
     nthreads = max(1, min(16, len(os.sched_getaffinity(0))))
     ftm = list(tbe.feature_table_map)
-    O.tbe_forward(store, ftm, B, new_ids, offs, psw, pooling, odt, "fbgemm", nthreads)  # warm-up / JIT
-    t0, reps = time.perf_counter(), 0
+    call = lambda i: O.tbe_forward(store, ftm, B, host[i][0], host[i][1], host[i][2], pooling, odt, "fbgemm", nthreads)
+    ref = call(0)  # warm-up (fbgemm generates its kernels on first use) and the output that is compared
+    t0, reps, done = time.perf_counter(), 0, 0
     while True:
-        ref = O.tbe_forward(store, ftm, B, new_ids, offs, psw, pooling, odt, "fbgemm", nthreads)
+        call(reps % NB)
+        done += host[reps % NB][0].size
         reps += 1
         el = time.perf_counter() - t0
-        if el > seconds or reps >= 200:
+        if el > seconds:
             break
-    L = ids.size
     got = out_gpu.cpu().numpy()
     if not wl["pooled"]:
         ref = ref[: got.shape[0]]  # rows of the first feature
     view = np.uint16 if got.dtype == np.float16 else np.uint32
     mism = int((got.view(view) != ref.view(view)).sum())
     return {
-        "value": L * reps / el,
+        "value": done / el,
         "unit": "lookups/s",
         "cores": nthreads,
         "kind": "reference",
-        "sample": f"batch 0 of the same workload ({L} lookups) x {reps} calls in {el:.1f} s; fbgemm "
-                  f"GenerateEmbeddingSpMDM[NBit]WithStrides from libtorch_cpu, bags split over {nthreads} threads, "
-                  f"tables compacted to the {int(sum(rows_t))} touched rows",
+        "sample": f"{reps} forwards over the same {NB} batches ({done} lookups) in {el:.1f} s; fbgemm "
+                  f"GenerateEmbeddingSpMDM[NBit]WithStrides from libtorch_cpu (the kernels behind the reference's CPU "
+                  f"TBE), bags split over {nthreads} threads; {where}",
         "gpu_vs_cpu_mismatching_outputs": mism,
         "outputs_compared": int(got.size),
     }
 
 
 # --------------------------------------------------------------------------
+# rocprofv3 output -> short text (the summaries kept under profiles/)
+# --------------------------------------------------------------------------
+def rocprof_summary(root):
+    import collections
+    import csv
+    import glob
+
+    mine = lambda name: "tbe_" in name or "tra_" in name or "tra::" in name
+    short = lambda name: name.split("(")[0].replace("void ", "")[:100]
+    for f in sorted(glob.glob(os.path.join(root, "**", "*kernel_stats.csv"), recursive=True)):
+        print(f"# {os.path.relpath(f, root)}")
+        print(f"{'calls':>8s} {'avg_us':>10s} {'min_us':>10s} {'max_us':>10s} {'pct':>7s}  kernel")
+        for r in csv.DictReader(open(f)):
+            if mine(r["Name"]):
+                print(f"{int(r['Calls']):8d} {float(r['AverageNs']) / 1e3:10.2f} {float(r['MinNs']) / 1e3:10.2f} "
+                      f"{float(r['MaxNs']) / 1e3:10.2f} {float(r['Percentage']):7.2f}  {short(r['Name'])}")
+    for f in sorted(glob.glob(os.path.join(root, "**", "*counter_collection.csv"), recursive=True)):
+        agg = collections.defaultdict(list)
+        for r in csv.DictReader(open(f)):
+            if mine(r["Kernel_Name"]):
+                agg[(short(r["Kernel_Name"]), r["Counter_Name"])].append(float(r["Counter_Value"]))
+        print(f"# {os.path.relpath(f, root)}")
+        print(f"{'dispatches':>10s} {'mean per dispatch':>20s}  counter  kernel")
+        for (k, c), v in sorted(agg.items()):
+            print(f"{len(v):10d} {sum(v) / len(v):20.1f}  {c}  {k}")
+
+
 def main():
     args = parse_args()
+    if args.rocprof_summary:
+        rocprof_summary(args.rocprof_summary)
+        return
     if args.row_alignment is None:
         args.row_alignment = 4 if args.config == "c5" else 16
     if args.gpus != 1:
@@ -373,6 +428,12 @@ def main():
     el = timed(args.mode, args.steps, args.warmup)
     other = "eager" if args.mode == "graph" else None
     el_other = timed("eager", args.steps, min(args.warmup, 50)) if other else None
+    # host-side cost of a step: the same loop without waiting for the GPU
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run("eager", min(args.steps, 500))
+    host_ms = (time.perf_counter() - t0) / min(args.steps, 500) * 1e3
+    torch.cuda.synchronize()
 
     # ---- kernel-only timing: the lookup launch(es) alone, HIP events on the launch stream
     tbe = module._emb_modules[0]
@@ -381,7 +442,14 @@ def main():
     from torchrec_amd import ops
     for v, l, w in batches:
         offs.append(ops.asynchronous_complete_cumsum(l))
-    kout = out_tensor(outs[0]).clone()
+    if wl["pooled"]:
+        kout = out_tensor(outs[0]).clone()
+    else:
+        # sequence lookup writes one row per id of every feature: [max L, D]
+        odt = torch.half if wl["out_dtype"] == torch.half else torch.float
+        kout = torch.empty(max(b[0].numel() for b in batches), wl["dims"][0], dtype=odt, device=dev)
+    if len(module._emb_modules) != 1:
+        raise RuntimeError("bench.py times one lookup operator; this workload built several")
     stream = _lib.current_stream(dev)
     plan = tbe._get_plan(None)
     pooling = int(tbe.pooling_mode)
@@ -393,7 +461,9 @@ def main():
         if rc != 0:
             _lib.check(rc)
 
-    n_launch_per_call = len(module._emb_modules[0]._plans) and 1
+    info = ctypes.create_string_buffer(4096)
+    _lib.check(lib.tra_tbe_launch_info(plan, wl["B"], batches[0][0].numel(), pooling, info, len(info)))
+    launches = info.value.decode().split("; ")
     for k in range(min(args.warmup, 200)):
         launch(k % NB)
     torch.cuda.synchronize()
@@ -407,6 +477,15 @@ def main():
     kernel_ms = e0.elapsed_time(e1) / ksteps
     alg = sum(wl["alg_bytes"][k % NB] for k in range(ksteps)) / ksteps
     achieved = alg / (kernel_ms * 1e-3) / 1e9
+
+    # A copy of known size by the library's own copy kernel: hardware-counter
+    # runs of this script read FETCH_SIZE / WRITE_SIZE for it next to the lookup.
+    cal = torch.empty(2, CAL_COPY_BYTES, dtype=torch.uint8, device=dev)
+    cal[0].fill_(1)
+    for _ in range(3):
+        _lib.check(lib.tra_copy_bytes(_lib.ptr(cal[0]), _lib.ptr(cal[1]), CAL_COPY_BYTES, stream))
+    torch.cuda.synchronize()
+    del cal
 
     traffic = None
     tpath = os.path.join(ROOT, "profiles", f"{args.config}_lookup_traffic.json")
@@ -444,12 +523,14 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
-            "kernel": "tbe_pooled_kernel" if wl["pooled"] else "tbe_nobag_kernel",
+            "kernel": launches[0].split(" ")[0],
+            "launches_per_call": launches,
             "kernel_ms": kernel_ms,
             "algorithmic_bytes_per_launch": alg,
             "kernel_lookups_per_s": (sum(lookups) / NB) / (kernel_ms * 1e-3),
         },
     }
+    result["host_enqueue_ms_per_step"] = host_ms
     if other:
         result["eager_value"] = total_lookups / el_other
         result["eager_ms_per_step"] = el_other / args.steps * 1e3

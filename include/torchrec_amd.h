@@ -110,6 +110,15 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
                     int32_t out_dtype, void* out, int64_t out_stride,
                     void* stream);
 
+/* Which kernels a tra_tbe_forward with these sizes launches, one entry per
+ * launch, "; "-separated, e.g. "tbe_pooled_cu_kernel dtype=int4 lane_bytes=8
+ * slices=26".  For profiling: the names are the ones a kernel trace shows.
+ * No counterpart in the reference: fbgemm_gpu picks its kernel inside the
+ * TBE module's forward (called at torchrec/quant/embedding_modules.py:547-557)
+ * and does not report it. */
+int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
+                        int32_t pooling_mode, char* buf, int32_t buf_len);
+
 /* Number of out-of-range ids seen by forwards on this plan since the last
  * call (synchronizes the stream; resets the counter).  Stands in for
  * fbgemm_gpu's bounds_check_indices. */
@@ -183,6 +192,13 @@ int tra_quantize_rows(const float* in, int64_t rows, int32_t dim, int32_t bits,
  * fp16 scale/bias at the END of each row. */
 int tra_quantize_rows_sbhalf(const float* in, int64_t rows, int32_t dim,
                              int32_t bits, uint8_t* out, void* stream);
+
+/* Measurement ------------------------------------------------------------- */
+/* Streaming device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte
+ * aligned pointers) by a kernel named tra_copy_kernel.  A copy of known size
+ * under the same hardware counters calibrates FETCH_SIZE / WRITE_SIZE readings
+ * of the lookup kernels.  No counterpart in the reference. */
+int tra_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

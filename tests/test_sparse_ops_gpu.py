@@ -13,7 +13,8 @@ pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
 
 
-@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 65, 4095, 4096, 4097, 100_003, 1_048_577])
+@pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 65, 2047, 2048, 2049, 4095, 4096, 4097, 53_248, 100_003,
+                               131_071, 131_072, 131_073, 1_048_577])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 def test_cumsum(n, dtype):
     rng = np.random.default_rng(n)
@@ -22,6 +23,17 @@ def test_cumsum(n, dtype):
     want = O.cumsum(lengths)
     assert got.dtype == want.dtype and np.array_equal(got, want)
     assert np.array_equal(want[1:], np.cumsum(lengths, dtype=dtype))  # closed form
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_cumsum_unaligned_view(dtype):
+    """Input that starts 4 (or 8) bytes into an allocation: no 16-byte loads."""
+    rng = np.random.default_rng(5)
+    lengths = rng.integers(0, 50, 20_001).astype(dtype)
+    view = torch.from_numpy(lengths).to(DEV)[1:]
+    assert view.data_ptr() % 16 != 0
+    got = ops.asynchronous_complete_cumsum(view).cpu().numpy()
+    assert np.array_equal(got, O.cumsum(lengths[1:]))
 
 
 def test_cumsum_int64_beyond_32_bits():

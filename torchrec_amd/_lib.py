@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = [
     "tra_tbe_create",
     "tra_tbe_destroy",
     "tra_tbe_forward",
+    "tra_tbe_launch_info",
     "tra_tbe_error_count",
     "tra_cumsum_workspace_bytes",
     "tra_cumsum",
@@ -34,6 +35,7 @@ EXPORTED_SYMBOLS = [
     "tra_bucketize_scatter",
     "tra_quantize_rows",
     "tra_quantize_rows_sbhalf",
+    "tra_copy_bytes",
 ]
 
 TRA_OK = 0
@@ -76,6 +78,7 @@ def lib() -> ctypes.CDLL:
         l.tra_tbe_create.argtypes = [ctypes.POINTER(TableSpec), i32, ctypes.POINTER(i32), ctypes.POINTER(i32), i32, ctypes.POINTER(vp)]
         l.tra_tbe_destroy.argtypes = [vp]
         l.tra_tbe_forward.argtypes = [vp, vp, vp, vp, i32, vp, i32, i64, i32, i32, vp, i64, vp]
+        l.tra_tbe_launch_info.argtypes = [vp, i32, i64, i32, ctypes.c_char_p, i32]
         l.tra_tbe_error_count.argtypes = [vp, vp, ctypes.POINTER(i64)]
         l.tra_cumsum_workspace_bytes.argtypes = [i64]
         l.tra_cumsum_workspace_bytes.restype = i64
@@ -87,6 +90,7 @@ def lib() -> ctypes.CDLL:
         l.tra_bucketize_scatter.argtypes = [vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp]
         l.tra_quantize_rows.argtypes = [vp, i64, i32, i32, vp, i32, vp]
         l.tra_quantize_rows_sbhalf.argtypes = [vp, i64, i32, i32, vp, vp]
+        l.tra_copy_bytes.argtypes = [vp, vp, i64, vp]
         _lib = l
     return _lib
 

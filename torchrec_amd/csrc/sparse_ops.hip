@@ -3,6 +3,8 @@
 // bit-exact by construction; these are bandwidth-trivial next to the gather.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
+
 #include "tra_common.h"
 
 namespace tra {
@@ -44,11 +46,79 @@ __global__ __launch_bounds__(kScanThreads) void tile_sums_kernel(const void* in,
                                                                   int64_t* sums) {
   __shared__ int64_t smem[kScanThreads / kWaveSize];
   const int64_t base = (int64_t)blockIdx.x * kScanTile;
+  int64_t x[kScanItems];
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    const int64_t i = base + k * kScanThreads + threadIdx.x;
+    x[k] = i < n ? ld<T>(in, i) : 0;
+  }
   int64_t v = 0;
-  for (int i = threadIdx.x; i < kScanTile; i += kScanThreads)
-    if (base + i < n) v += ld<T>(in, base + i);
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) v += x[k];
   v = block_sum(v, smem);
   if (threadIdx.x == 0) sums[blockIdx.x] = v;
+}
+
+// One-launch variant for short inputs: every block first sums everything in
+// front of its tile (redundant reads, a few hundred KB from L2 at most), then
+// scans the tile.  Tiles are kSmallThreads * (16 / sizeof(T)) elements.
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallMaxTiles = 64;
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kSmallThreads) void scan_small_kernel(const T* __restrict__ in,
+                                                                    int64_t n, T* __restrict__ out) {
+  constexpr int V = 16 / (int)sizeof(T);
+  struct __align__(16) Vec { T v[V]; };
+  __shared__ int64_t smem[kSmallThreads / kWaveSize];
+  __shared__ int64_t wave_tot[kSmallThreads / kWaveSize];
+  const int t = threadIdx.x;
+  int64_t pre = 0;
+  if (VEC) {
+    const Vec* vin = reinterpret_cast<const Vec*>(in);
+#pragma unroll 4
+    for (int k = 0; k < (int)blockIdx.x; ++k) {
+      const Vec x = vin[(int64_t)k * kSmallThreads + t];
+#pragma unroll
+      for (int i = 0; i < V; ++i) pre += (int64_t)x.v[i];
+    }
+  } else {
+#pragma unroll 4
+    for (int k = 0; k < (int)blockIdx.x * V; ++k) pre += (int64_t)in[(int64_t)k * kSmallThreads + t];
+  }
+  pre = block_sum(pre, smem);
+  const int64_t base = ((int64_t)blockIdx.x * kSmallThreads + t) * V;
+  int64_t x[V];
+  if (VEC && base + V <= n) {
+    const Vec q = reinterpret_cast<const Vec*>(in)[base / V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) x[i] = (int64_t)q.v[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < V; ++i) x[i] = base + i < n ? (int64_t)in[base + i] : 0;
+  }
+  int64_t tsum = 0;
+#pragma unroll
+  for (int i = 0; i < V; ++i) tsum += x[i];
+  const int lane = t & (kWaveSize - 1);
+  const int wave = t / kWaveSize;
+  int64_t inc = tsum;
+#pragma unroll
+  for (int off = 1; off < kWaveSize; off <<= 1) {
+    const int64_t o = __shfl_up(inc, off, 64);
+    if (lane >= off) inc += o;
+  }
+  if (lane == kWaveSize - 1) wave_tot[wave] = inc;
+  __syncthreads();
+  int64_t wprefix = 0;
+  for (int w = 0; w < wave; ++w) wprefix += wave_tot[w];
+  int64_t run = pre + wprefix + inc - tsum;
+  if (blockIdx.x == 0 && t == 0) out[0] = 0;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    run += x[i];
+    if (base + i < n) out[base + i + 1] = (T)run;
+  }
 }
 
 template <typename T>
@@ -243,6 +313,14 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* in, int
   }
 }
 
+// Plain streaming copy, 16 bytes per lane per step.
+__global__ __launch_bounds__(256) void tra_copy_kernel(const uint4* __restrict__ src,
+                                                        uint4* __restrict__ dst, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+    dst[i] = src[i];
+}
+
 static int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e, what);
@@ -285,7 +363,11 @@ using namespace tra;
 
 extern "C" {
 
+// Longest input the one-launch scan takes (64 tiles of int64, 32 of int32).
+constexpr int64_t kSmallScanMax = (int64_t)kSmallMaxTiles * kSmallThreads * 2;
+
 int64_t tra_cumsum_workspace_bytes(int64_t n) {
+  if (n <= kSmallScanMax) return 0;
   const int64_t tiles = (n + kScanTile - 1) / kScanTile;
   return tiles > 1 ? tiles * (int64_t)sizeof(int64_t) : 0;
 }
@@ -301,6 +383,27 @@ int tra_cumsum(const void* lengths, int64_t n, int32_t is_i64, void* offsets, vo
     return TRA_ERR_TOO_LARGE;
   }
   hipStream_t s = (hipStream_t)stream;
+  if (n <= kSmallScanMax) {
+    const int per_tile = kSmallThreads * (is_i64 ? 2 : 4);
+    const unsigned g = (unsigned)std::max<int64_t>(1, (n + per_tile - 1) / per_tile);
+    const bool vec = (uintptr_t)lengths % 16 == 0;
+    if (is_i64) {
+      if (vec)
+        hipLaunchKernelGGL((scan_small_kernel<int64_t, true>), dim3(g), dim3(kSmallThreads), 0, s,
+                           (const int64_t*)lengths, n, (int64_t*)offsets);
+      else
+        hipLaunchKernelGGL((scan_small_kernel<int64_t, false>), dim3(g), dim3(kSmallThreads), 0, s,
+                           (const int64_t*)lengths, n, (int64_t*)offsets);
+    } else {
+      if (vec)
+        hipLaunchKernelGGL((scan_small_kernel<int32_t, true>), dim3(g), dim3(kSmallThreads), 0, s,
+                           (const int32_t*)lengths, n, (int32_t*)offsets);
+      else
+        hipLaunchKernelGGL((scan_small_kernel<int32_t, false>), dim3(g), dim3(kSmallThreads), 0, s,
+                           (const int32_t*)lengths, n, (int32_t*)offsets);
+    }
+    return check_launch("tra_cumsum");
+  }
   const int64_t tiles = n == 0 ? 1 : (n + kScanTile - 1) / kScanTile;
   int64_t* sums = nullptr;
   if (tiles > 1) {
@@ -457,6 +560,23 @@ int tra_quantize_rows_sbhalf(const float* in, int64_t rows, int32_t dim, int32_t
                              uint8_t* out, void* stream) {
   const int64_t rb = bits > 0 && bits <= 8 ? (int64_t)dim * bits / 8 + 4 : 0;
   return quantize_impl(in, rows, dim, bits, out, rb, 0, (hipStream_t)stream);
+}
+
+int tra_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream) {
+  if (bytes < 0 || bytes % 16 != 0 || (uintptr_t)src % 16 != 0 || (uintptr_t)dst % 16 != 0) {
+    set_error("tra_copy_bytes: size and pointers must be multiples of 16 bytes");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (bytes == 0) return TRA_OK;
+  if (!src || !dst) {
+    set_error("tra_copy_bytes: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int64_t n16 = bytes / 16;
+  const unsigned grid = (unsigned)std::min<int64_t>((n16 + 255) / 256, 256 * 32);
+  hipLaunchKernelGGL(tra_copy_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4*)src, (uint4*)dst, n16);
+  return check_launch("tra_copy_bytes");
 }
 
 }  // extern "C"

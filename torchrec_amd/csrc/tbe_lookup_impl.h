@@ -33,6 +33,7 @@ struct SubClass {
   int32_t lpr;             // lanes per row
   int32_t tiles_per_feat;  // blocks per feature
   int32_t tile_start;      // first block of this sub-class in the grid
+  int32_t window;          // window kernel: bags per block
 };
 
 struct LookupArgs {
@@ -51,7 +52,6 @@ struct LookupArgs {
   int32_t mean;
   int32_t vec_store;  // 1: every lane's output slice is 16-byte aligned
   int32_t out_fp16;
-  int32_t window_bags;  // balanced pooled kernel: bags per block
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
   int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
 #ifdef TRA_INSTRUMENT
@@ -511,9 +511,9 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     if (i < a.n_sub && blk >= a.sub[i].tile_start) s = i;
   const SubClass sc = a.sub[s];
   const int nb_all = sc.count * a.B;
-  const int q0 = (blk - sc.tile_start) * a.window_bags;
+  const int q0 = (blk - sc.tile_start) * sc.window;
   if (q0 >= nb_all) return;
-  const int nb = min(a.window_bags, nb_all - q0);
+  const int nb = min(sc.window, nb_all - q0);
 
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
   __syncthreads();

@@ -1,6 +1,7 @@
 // Host side of the TBE lookup: plan construction (tra_tbe_create) and launch
 // (tra_tbe_forward), plus the small library-level entry points.
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -254,6 +255,43 @@ int tra_tbe_destroy(tra_tbe_t tbe) {
   return TRA_OK;
 }
 
+// Whether a pooled call goes to the per-CU window kernel: the size heuristic
+// (or its override) and the limits of the kernel's packed window entries.
+static bool use_window_kernel(const tra_tbe* tbe, const Tuning& tune, bool nobag,
+                              int32_t batch_size) {
+  bool balanced = !nobag && tune.balanced && batch_size <= (1 << kBagBits);
+  for (const FeatureDesc& d : tbe->slices)
+    if (d.feature > 32767) balanced = false;
+  for (const LaunchClass& cls : tbe->classes)
+    if ((int64_t)cls.feats.size() >= (int64_t(1) << (32 - kBagBits)) ||
+        (int64_t)cls.feats.size() * batch_size >= (int64_t(1) << 31))
+      balanced = false;
+  return balanced;
+}
+
+int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
+                        int32_t pooling_mode, char* buf, int32_t buf_len) {
+  if (!tbe || !buf || buf_len <= 0) {
+    set_error("tra_tbe_launch_info: null argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const bool nobag = pooling_mode == TRA_POOL_NONE;
+  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
+  const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
+  static const char* const kDtypeName[] = {"fp32", "fp16", "int8", "int4", "int2"};
+  std::string text;
+  for (const LaunchClass& cls : tbe->classes) {
+    char line[160];
+    snprintf(line, sizeof(line), "%s%s dtype=%s lane_bytes=%d slices=%d",
+             text.empty() ? "" : "; ",
+             nobag ? "tbe_nobag_kernel" : (balanced ? "tbe_pooled_cu_kernel" : "tbe_pooled_kernel"),
+             kDtypeName[cls.dtype], cls.cb, (int)cls.feats.size());
+    text += line;
+  }
+  snprintf(buf, (size_t)buf_len, "%s", text.c_str());
+  return TRA_OK;
+}
+
 int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
                     const void* offsets, int32_t idx_is_i64, const float* per_sample_weights,
                     int32_t batch_size, int64_t num_indices, int32_t pooling_mode,
@@ -292,13 +330,7 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
   const int esz = out_dtype == TRA_FP16 ? 2 : 4;
   hipStream_t s = (hipStream_t)stream;
   const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
-  bool balanced = !nobag && tune.balanced && batch_size <= (1 << kBagBits);
-  for (const FeatureDesc& d : tbe->slices)
-    if (d.feature > 32767) balanced = false;
-  for (const LaunchClass& cls : tbe->classes)
-    if ((int64_t)cls.feats.size() >= (int64_t(1) << (32 - kBagBits)) ||
-        (int64_t)cls.feats.size() * batch_size >= (int64_t(1) << 31))
-      balanced = false;
+  const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
   for (const LaunchClass& cls : tbe->classes) {
     LookupArgs a;
     memset(&a, 0, sizeof(a));
@@ -327,18 +359,39 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
     if (!nobag)
       for (int id : cls.feats) vec = vec && ((int64_t)tbe->slices[id].out_col * esz % 16 == 0);
     a.vec_store = vec;
-    int window = 0;
+    // Window kernel: every block should get about the same amount of work, so
+    // a sub-class's window (bags per block) shrinks with its row width.  A
+    // row costs its payload bytes, but never less than 256: below that the
+    // per-row requests (id, header, one line) dominate and rows of any width
+    // take the same time.  Aim at one block per CU; more passes when a window
+    // would not fit the kernel's LDS arrays.
+    const int64_t cost_floor = env_int("TRA_COST_FLOOR", 256);
+    auto bag_cost = [&](size_t i) { return std::max<int64_t>((int64_t)cls.lprs[i] * cls.cb, cost_floor); };
+    int64_t work_per_block = 0;
     if (balanced) {
-      // One window per CU when that fits the LDS arrays, else several per CU.
-      window = tune.window;
-      if (window == 0) {
-        const int64_t class_bags = (int64_t)cls.feats.size() * batch_size;
-        const int64_t per_cu = (class_bags + kNumCus - 1) / kNumCus;
-        const int64_t passes = (per_cu + kMaxWindow - 1) / kMaxWindow;
-        window = (int)((per_cu + passes - 1) / passes);
-        if (window < 64) window = 64;
+      int64_t total = 0, min_cost = INT64_MAX;
+      for (size_t i = 0; i < cls.feats.size(); ++i) {
+        total += (int64_t)batch_size * bag_cost(i);
+        min_cost = std::min(min_cost, bag_cost(i));
       }
-      a.window_bags = window;
+      int64_t blocks = kNumCus;
+      while ((total + blocks - 1) / blocks > (int64_t)kMaxWindow * min_cost) blocks += kNumCus;
+      work_per_block = (total + blocks - 1) / blocks;
+      // Rounding each sub-class up to whole windows must not spill a few
+      // blocks into an extra pass: grow the share until the grid fits.
+      for (int iter = 0; iter < 64; ++iter) {
+        int64_t g = 0;
+        for (size_t i = 0; i < cls.feats.size();) {
+          size_t j = i;
+          while (j < cls.feats.size() && cls.lprs[j] == cls.lprs[i]) ++j;
+          const int64_t w = std::max<int64_t>(
+              64, std::min<int64_t>((work_per_block + bag_cost(i) - 1) / bag_cost(i), kMaxWindow));
+          g += ((int64_t)(j - i) * batch_size + w - 1) / w;
+          i = j;
+        }
+        if (g <= blocks) break;
+        work_per_block += std::max<int64_t>(1, work_per_block / 128);
+      }
       for (size_t i = 0; i < cls.feats.size() && i < (size_t)kMaxPos; ++i)
         a.feat_pos[i] = (int16_t)tbe->slices[cls.feats[i]].feature;
     }
@@ -363,7 +416,10 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
         grid += sc.count * sc.tiles_per_feat;
       } else if (balanced) {
         const int64_t nb = (int64_t)sc.count * batch_size;
+        int64_t window = tune.window > 0 ? tune.window : (work_per_block + bag_cost(i) - 1) / bag_cost(i);
+        window = std::max<int64_t>(64, std::min<int64_t>(window, kMaxWindow));
         sc.tiles_per_feat = 0;
+        sc.window = (int)window;
         grid += (int)((nb + window - 1) / window);
       } else {
         sc.tiles_per_feat = (batch_size + per_block - 1) / per_block;
