@@ -110,6 +110,27 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
                     int32_t out_dtype, void* out, int64_t out_stride,
                     void* stream);
 
+/* The same lookup from the KJT's lengths instead of its offsets: what
+ * QuantEmbeddingBagCollection.forward does when the KJT was built from
+ * lengths, i.e. KeyedJaggedTensor.offsets() -> asynchronous_complete_cumsum
+ * (torchrec/sparse/jagged_tensor.py:101-107, 79-80) followed by the TBE call
+ * (torchrec/quant/embedding_modules.py:547-557), in one entry point.
+ *   lengths      device [num_keys * batch_size], same integer type as indices
+ *   num_keys     number of keys of the KJT (>= every feature position + 1)
+ *   workspace    device scratch of tra_tbe_forward_lengths_workspace_bytes()
+ *                bytes; contents unspecified afterwards
+ * Large pooled calls derive each bag's start inside the lookup kernel (no
+ * offsets array is produced); all others run tra_cumsum into the workspace
+ * and then the ordinary lookup.  Results are those of tra_tbe_forward. */
+int64_t tra_tbe_forward_lengths_workspace_bytes(int32_t num_keys, int32_t batch_size,
+                                                int32_t idx_is_i64);
+int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indices,
+                            const void* lengths, int32_t idx_is_i64,
+                            const float* per_sample_weights, int32_t batch_size,
+                            int32_t num_keys, int64_t num_indices,
+                            int32_t pooling_mode, int32_t out_dtype, void* out,
+                            int64_t out_stride, void* workspace, void* stream);
+
 /* Which kernels a tra_tbe_forward with these sizes launches, one entry per
  * launch, "; "-separated, e.g. "tbe_pooled_cu_kernel dtype=int4 lane_bytes=8
  * slices=26".  For profiling: the names are the ones a kernel trace shows.

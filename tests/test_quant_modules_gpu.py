@@ -212,3 +212,33 @@ def test_empty_batch_and_empty_features():
                             lengths=torch.zeros(4, dtype=torch.int32, device=DEV))
     out = q(kjt).values()
     assert out.shape == (4, 16) and not out.any()
+
+
+def test_qebc_kjt_from_lengths_equals_from_offsets():
+    """A KJT built from lengths (the operator derives the offsets) and the same
+    KJT built from offsets give identical KeyedTensors."""
+    import numpy as np
+    from torchrec_amd import KeyedJaggedTensor
+    from torchrec_amd.modules.embedding_configs import DataType, EmbeddingBagConfig, PoolingType
+    from torchrec_amd.quant import EmbeddingBagCollection as QuantEBC
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(3)
+    T, B = 5, 64
+    tables = [EmbeddingBagConfig(name=f"t{t}", embedding_dim=32, num_embeddings=500 + t, feature_names=[f"f{t}"],
+                                 data_type=DataType.INT4, pooling=PoolingType.SUM) for t in range(T)]
+    m = QuantEBC(tables, False, dev, output_dtype=torch.float)
+    for tbe in m._emb_modules:
+        tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, device=dev))
+        for t in range(len(tbe.rows)):  # finite fp16 scale/bias headers
+            v = tbe._rows_view(t)
+            v[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=dev)
+    lengths = torch.randint(0, 9, (T * B,), dtype=torch.int32, device=dev)
+    values = torch.randint(0, 500, (int(lengths.sum()),), dtype=torch.int32, device=dev)
+    keys = [f"f{t}" for t in range(T)]
+    a = m(KeyedJaggedTensor(keys=keys, values=values, lengths=lengths))
+    offsets = torch.zeros(T * B + 1, dtype=torch.int32, device=dev)
+    offsets[1:] = torch.cumsum(lengths, 0)
+    b = m(KeyedJaggedTensor(keys=keys, values=values, offsets=offsets))
+    assert a.keys() == b.keys() and torch.equal(a.values(), b.values())
+    assert torch.isfinite(a.values()).all()

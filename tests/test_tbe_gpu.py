@@ -352,3 +352,79 @@ def test_lookup_under_hip_graph():
         want = O.tbe_forward(store, list(range(T)), B, i, o, None, O.SUM, O.FP16)
         assert bits_equal(got, want) == 0, seed
         assert bits_equal(eager, want) == 0, seed
+
+
+def _from_lengths(tbe, ids, lengths, psw, B, **kw):
+    return tbe(torch.from_numpy(ids).to(DEV), None, None if psw is None else torch.from_numpy(psw).to(DEV),
+               lengths=torch.from_numpy(lengths).to(DEV), batch_size=B, **kw).cpu().numpy()
+
+
+@pytest.mark.parametrize("window", [None, 64, 100, 0, 2048])
+@pytest.mark.parametrize("dtype,pooling,weighted,idt", [
+    (O.INT4, O.SUM, False, np.int32), (O.INT8, O.MEAN, True, np.int64), (O.FP16, O.SUM, True, np.int32),
+    (O.INT2, O.MEAN, False, np.int64), (O.FP32, O.SUM, False, np.int32)])
+def test_forward_from_lengths(monkeypatch, window, dtype, pooling, weighted, idt):
+    """forward(offsets=None, lengths=...) against the oracle: the small-call route
+    (scan + lookup, window None) and the window kernel deriving the bag starts
+    itself, with windows that span feature boundaries."""
+    if window is not None:
+        monkeypatch.setenv("TRA_BALANCED", "1")
+        monkeypatch.setenv("TRA_WINDOW", str(window))
+    rng = np.random.default_rng(300 + dtype + pooling + (window or 7))
+    rows, B, dim = 3000, 211, 64
+    specs = [(dtype, rows, dim), (dtype, rows + 13, dim), (dtype, rows + 5, dim)]
+    ftm = [0, 1, 2, 0, 1]
+    tbe, store = build(rng, specs, ftm, pooling, O.FP32, 16)
+    rows_f = [specs[t][1] for t in ftm]
+    lengths, offsets, ids = make_bags(rng, rows_f, B, 50, idt)
+    psw = rng.uniform(-1, 1, len(ids)).astype(np.float32) if weighted else None
+    want = O.tbe_forward(store, ftm, B, ids, offsets, psw, pooling, O.FP32)
+    got = _from_lengths(tbe, ids, lengths, psw, B)
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
+
+
+def test_forward_from_lengths_scattered_keys(monkeypatch):
+    """Window kernel from lengths when the operator's features sit at scattered,
+    descending and repeated-gap key positions of a wider KJT (every feature
+    boundary inside a window starts a new run), plus an int64 total beyond the
+    first features and empty leading keys."""
+    monkeypatch.setenv("TRA_BALANCED", "1")
+    monkeypatch.setenv("TRA_WINDOW", "150")
+    rng = np.random.default_rng(17)
+    rows, B, dim = 900, 97, 128
+    specs = [(O.INT4, rows, dim)] * 4
+    tbe, store = build(rng, specs, [0, 1, 2, 3], O.SUM, O.FP16, 16)
+    K = 7
+    positions = [5, 2, 3, 0]           # keys 1, 4, 6 unused; 2 -> 3 is the only adjacent pair
+    lengths, offsets, ids = make_bags(rng, [rows] * K, B, 30)
+    got = _from_lengths(tbe, ids, lengths, None, B, feature_positions=positions)
+    seg = [ids[offsets[k * B]:offsets[(k + 1) * B]] for k in range(K)]
+    Lm = lengths.reshape(K, B)
+    o_off = np.zeros(4 * B + 1, dtype=np.int32)
+    o_off[1:] = np.cumsum(np.concatenate([Lm[p] for p in positions]))
+    want = O.tbe_forward(store, [0, 1, 2, 3], B, np.concatenate([seg[p] for p in positions]), o_off, None, O.SUM, O.FP16)
+    assert bits_equal(got, want) == 0
+    # same through the offsets entry point
+    got2 = tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV), feature_positions=positions,
+               batch_size=B).cpu().numpy()
+    assert bits_equal(got2, want) == 0
+    # an unaligned lengths view takes the scan + lookup route and gives the same bits
+    padded = torch.zeros(len(lengths) + 1, dtype=torch.int32, device=DEV)
+    padded[1:] = torch.from_numpy(lengths)
+    assert padded[1:].data_ptr() % 16 != 0
+    got3 = tbe(torch.from_numpy(ids).to(DEV), None, lengths=padded[1:], feature_positions=positions,
+               batch_size=B).cpu().numpy()
+    assert bits_equal(got3, want) == 0
+
+
+def test_forward_from_lengths_at_scale():
+    """Default routing at 26 x 2048 bags (~1M ids): lengths entry == offsets entry, bit for bit."""
+    rng = np.random.default_rng(2025)
+    T, rows, dim, B = 26, 50_000, 128, 2048
+    tbe, store = build(rng, [(O.INT4, rows, dim)] * T, list(range(T)), O.SUM, O.FP16, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 40, empty_frac=0.05)
+    ti = torch.from_numpy(ids).to(DEV)
+    a = tbe(ti, torch.from_numpy(offsets).to(DEV))
+    b = tbe(ti, None, lengths=torch.from_numpy(lengths).to(DEV), batch_size=B)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))

@@ -489,7 +489,67 @@ __device__ __forceinline__ int length_bin(int len) {
   return len < 192 ? len : min(kLenBins - 1, 192 + ((len - 192) >> 6));
 }
 
-template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U>
+// Accumulator of the from-lengths prologue: as wide as the index type (with
+// int32 offsets every partial sum fits 32 bits by definition).
+template <typename IdxT>
+struct SumOf { using type = int64_t; };
+template <>
+struct SumOf<int32_t> { using type = int32_t; };
+
+// This thread's share of sum(lengths[0 .. p)): the block reads the range 16
+// bytes per lane per step, eight independent loads at a time (indices past the
+// end are clamped and their values dropped, so no load is predicated).  Every
+// block of the grid reads a prefix of the same array at the same moment, so
+// each starts at a different 16 KB step (`rot`) to spread the L2 channels.
+// `lengths` is 16-byte aligned.
+template <typename IdxT>
+__device__ __forceinline__ typename SumOf<IdxT>::type prefix_partial(const IdxT* __restrict__ lengths,
+                                                                     int64_t p, int rot) {
+  using S = typename SumOf<IdxT>::type;
+  constexpr int V = 16 / (int)sizeof(IdxT);
+  struct __align__(16) Vec { IdxT v[V]; };
+  const Vec* vin = reinterpret_cast<const Vec*>(lengths);
+  const int nvec = (int)(p / V);
+  const int nk = (nvec + kCuThreads - 1) / kCuThreads;
+  S part = 0;
+  for (int k0 = 0; k0 < nk; k0 += 8) {
+    Vec x[8];
+    int idx[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      idx[k] = ((k0 + k + rot) % nk) * kCuThreads + (int)threadIdx.x;
+      x[k] = vin[min(idx[k], nvec - 1)];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      S sum = 0;
+#pragma unroll
+      for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
+      part += (k0 + k < nk && idx[k] < nvec) ? sum : (S)0;
+    }
+  }
+  if ((int64_t)threadIdx.x < p - (int64_t)nvec * V) part += (S)lengths[(int64_t)nvec * V + threadIdx.x];
+  return part;
+}
+
+template <typename S>
+__device__ __forceinline__ S wave_total_t(S v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWaveSize);
+  return v;
+}
+
+// Position of feature `fi` of a sub-class among the input keys: from the launch
+// arguments when the class is small enough, else from the descriptors.
+__device__ __forceinline__ int feat_key_pos(const LookupArgs& a, const SubClass& sc, int fi) {
+  return sc.first + fi < kMaxPos ? (int)a.feat_pos[sc.first + fi]
+                                 : a.descs[a.feats[sc.first + fi]].feature;
+}
+
+// FROM_LENGTHS: a.offsets points at the KJT's lengths instead of its offsets
+// and the block derives its bags' start positions itself: one block-wide sum
+// of everything in front of the window plus a scan of the window in LDS.
+template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, bool FROM_LENGTHS = false>
 __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;
   extern __shared__ unsigned char tra_dyn_smem[];  // only its size matters (one block per CU)
@@ -515,25 +575,104 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   if (q0 >= nb_all) return;
   const int nb = min(sc.window, nb_all - q0);
 
+  // From lengths: the loads for the total in front of the window go out first,
+  // so that they share one memory latency with the loads of the window itself.
+  const int fi_lo = q0 / a.B;
+  using Sum = typename SumOf<IdxT>::type;
+  Sum front_part = 0;
+  if (FROM_LENGTHS)
+    front_part = prefix_partial<IdxT>(reinterpret_cast<const IdxT*>(a.offsets),
+                                      (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B), blk);
+
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < nb; i += kCuThreads) {
     const int q = q0 + i;
     const int fi = q / a.B;
     const int b = q - fi * a.B;
-    // Position of the bag's feature among the input keys: from the launch
-    // arguments when the class is small enough, else from the descriptors.
-    const int fpos = sc.first + fi < kMaxPos ? (int)a.feat_pos[sc.first + fi]
-                                             : a.descs[a.feats[sc.first + fi]].feature;
+    const int fpos = feat_key_pos(a, sc, fi);
     const int64_t bag = (int64_t)fpos * a.B + b;
-    const int64_t st = load_index<IdxT>(a.offsets, bag);
-    s_start[i] = st;
-    const int len = max(0, (int)(load_index<IdxT>(a.offsets, bag + 1) - st));
+    int len;
+    if (FROM_LENGTHS) {
+      len = max(0, (int)load_index<IdxT>(a.offsets, bag));
+    } else {
+      const int64_t st = load_index<IdxT>(a.offsets, bag);
+      s_start[i] = st;
+      len = max(0, (int)(load_index<IdxT>(a.offsets, bag + 1) - st));
+    }
     s_len[i] = len;
     s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
     s_slot[i] = (uint16_t)atomicAdd(&s_hist[length_bin(len)], 1);
   }
   __syncthreads();
+  if (FROM_LENGTHS) {
+    __shared__ Sum s_red[kCuWaves];
+    __shared__ Sum s_wave_tot[kCuWaves];
+    const int t = threadIdx.x;
+    const int wv = t / kWaveSize;
+    const int ln = t & (kWaveSize - 1);
+    // Exclusive scan of the window's lengths (window order): two bags per
+    // thread, wave scan, then the 16 wave totals.  The same barrier carries
+    // the block-wide total of everything in front of the window.
+    const Sum x0 = 2 * t < nb ? s_len[2 * t] : 0;
+    const Sum x1 = 2 * t + 1 < nb ? s_len[2 * t + 1] : 0;
+    Sum inc = x0 + x1;
+#pragma unroll
+    for (int off = 1; off < kWaveSize; off <<= 1) {
+      const Sum o = __shfl_up(inc, off, kWaveSize);
+      if (ln >= off) inc += o;
+    }
+    const Sum front_w = wave_total_t<Sum>(front_part);
+    if (ln == kWaveSize - 1) s_wave_tot[wv] = inc;
+    if (ln == 0) s_red[wv] = front_w;
+    __syncthreads();
+    Sum before = 0, front = 0;
+#pragma unroll
+    for (int w = 0; w < kCuWaves; ++w) {
+      if (w < wv) before += s_wave_tot[w];
+      front += s_red[w];
+    }
+    const Sum excl = before + inc - (x0 + x1);
+    // The window covers bags of features fi_lo .. fi_hi of the sub-class.  A
+    // feature's bags are contiguous in `lengths`; where the next feature's
+    // key position follows directly, the run simply continues.
+    const int fi_hi = (q0 + nb - 1) / a.B;
+    bool one_run = true;
+    for (int fi = fi_lo; fi < fi_hi; ++fi) one_run = one_run && feat_key_pos(a, sc, fi + 1) == feat_key_pos(a, sc, fi) + 1;
+    if (one_run) {
+      if (2 * t < nb) s_start[2 * t] = (int64_t)(front + excl);
+      if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(front + excl + x0);
+      __syncthreads();
+    } else {
+      // General case: keep the bare scan, then add to each run what lies in
+      // front of it (summed again for every run that does not continue the
+      // previous one).
+      if (2 * t < nb) s_start[2 * t] = (int64_t)excl;
+      if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(excl + x0);
+      __syncthreads();
+      int64_t adj = (int64_t)front;  // start = adj + scan value, for the current run
+      int64_t next_pos = -1;
+      for (int fi = fi_lo; fi <= fi_hi; ++fi) {
+        const int first = max(0, fi * a.B - q0);        // first bag of this feature in the window
+        const int last = min(nb, (fi + 1) * a.B - q0);  // one past its last bag
+        const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * a.B + (q0 + first - fi * a.B);
+        if (fi != fi_lo && pos != next_pos) {
+          const Sum w_ = wave_total_t<Sum>(
+              prefix_partial<IdxT>(reinterpret_cast<const IdxT*>(a.offsets), pos, blk));
+          if (ln == 0) s_red[wv] = w_;
+          __syncthreads();
+          Sum total = 0;
+#pragma unroll
+          for (int w = 0; w < kCuWaves; ++w) total += s_red[w];
+          adj = (int64_t)total - s_start[first];
+        }
+        next_pos = pos + (last - first);
+        __syncthreads();  // s_red and s_start[first] have been read by everyone
+        for (int i = first + t; i < last; i += kCuThreads) s_start[i] += adj;
+        __syncthreads();
+      }
+    }
+  }
   TRA_STAMP(1);
   // Counting sort, longest first: a permutation of 0..nb-1.  hist[] holds the
   // bin sizes and every bag already has its slot within its bin; one wave
@@ -670,6 +809,7 @@ struct LaunchParams {
   bool idx64;
   bool weighted;
   bool nobag;
+  bool from_lengths;  // window kernel reads lengths and derives offsets itself
 };
 
 template <int DTYPE>
@@ -684,7 +824,10 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
   }
 #define TRA_POOLED(W, U)                                                                       \
   do {                                                                                         \
-    if (p.balanced)                                                                            \
+    if (p.balanced && p.from_lengths)                                                          \
+      hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, 4, true>), g,               \
+                         dim3(kCuThreads), p.lds_bytes, stream, a);                            \
+    else if (p.balanced)                                                                       \
       hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kCuThreads),   \
                          p.lds_bytes, stream, a);                                              \
     else                                                                                       \

@@ -292,10 +292,33 @@ int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
   return TRA_OK;
 }
 
-int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
-                    const void* offsets, int32_t idx_is_i64, const float* per_sample_weights,
-                    int32_t batch_size, int64_t num_indices, int32_t pooling_mode,
-                    int32_t out_dtype, void* out, int64_t out_stride, void* stream) {
+// Largest number of features one window of the from-lengths kernel may span.
+constexpr int kMaxWindowFeatures = 32;
+
+// Can a pooled call with these sizes take the window kernel in its
+// from-lengths form (which needs no offsets)?
+static bool fused_scan_possible(const tra_tbe* tbe, int32_t batch_size, int32_t num_keys,
+                                int64_t num_indices, int32_t pooling_mode, const void* lengths) {
+  if (pooling_mode == TRA_POOL_NONE || batch_size <= 0 || tbe->num_features == 0) return false;
+  if ((uintptr_t)lengths % 16 != 0) return false;
+  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
+  if (!use_window_kernel(tbe, tune, false, batch_size)) return false;
+  const int fused = env_int("TRA_FUSED_SCAN", -1);
+  if (fused >= 0) return fused != 0;
+  // A window of up to kMaxWindow bags spans kMaxWindow / B + 2 features at most.
+  if (kMaxWindow / batch_size + 2 > kMaxWindowFeatures) return false;
+  // Every block of every launch sums the lengths in front of its window
+  // (about 1.3 us + 1 us per 40k lengths, measured); a separate scan costs
+  // about 7 us once.  Take whichever is less.
+  const int64_t n = (int64_t)num_keys * batch_size;
+  return (int64_t)tbe->classes.size() * (13 + n / 4000) < 70;
+}
+
+static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
+                        const void* offsets, bool from_lengths, int32_t idx_is_i64,
+                        const float* per_sample_weights, int32_t batch_size, int64_t num_indices,
+                        int32_t pooling_mode, int32_t out_dtype, void* out, int64_t out_stride,
+                        void* stream) {
   if (!tbe) {
     set_error("tra_tbe_forward: null plan");
     return TRA_ERR_INVALID_ARGUMENT;
@@ -441,6 +464,7 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
     lp.idx64 = idx_is_i64 != 0;
     lp.weighted = a.psw != nullptr;
     lp.nobag = nobag;
+    lp.from_lengths = from_lengths;
     int rc;
     switch (cls.dtype) {
       case TRA_INT8: rc = launch_lookup<TRA_INT8>(a, cls.cb, lp, s); break;
@@ -452,6 +476,63 @@ int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
     if (rc != TRA_OK) return rc;
   }
   return TRA_OK;
+}
+
+int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
+                    const void* offsets, int32_t idx_is_i64, const float* per_sample_weights,
+                    int32_t batch_size, int64_t num_indices, int32_t pooling_mode,
+                    int32_t out_dtype, void* out, int64_t out_stride, void* stream) {
+  return forward_impl(tbe, weights, indices, offsets, false, idx_is_i64, per_sample_weights,
+                      batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream);
+}
+
+int64_t tra_tbe_forward_lengths_workspace_bytes(int32_t num_keys, int32_t batch_size,
+                                                int32_t idx_is_i64) {
+  if (num_keys < 0 || batch_size < 0) return 0;
+  const int64_t n = (int64_t)num_keys * batch_size;
+  const int64_t off_bytes = ((n + 1) * (idx_is_i64 ? 8 : 4) + 255) / 256 * 256;
+  return off_bytes + tra_cumsum_workspace_bytes(n);
+}
+
+int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indices,
+                            const void* lengths, int32_t idx_is_i64,
+                            const float* per_sample_weights, int32_t batch_size, int32_t num_keys,
+                            int64_t num_indices, int32_t pooling_mode, int32_t out_dtype, void* out,
+                            int64_t out_stride, void* workspace, void* stream) {
+  if (!tbe) {
+    set_error("tra_tbe_forward_lengths: null plan");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (num_keys < 0 || batch_size < 0 || num_indices < 0) {
+    set_error("tra_tbe_forward_lengths: negative size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  for (const FeatureDesc& d : tbe->slices)
+    if (d.feature >= num_keys) {
+      set_error("tra_tbe_forward_lengths: feature position %d but only %d keys", d.feature,
+                num_keys);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+  if (!lengths && (int64_t)num_keys * batch_size > 0) {
+    set_error("tra_tbe_forward_lengths: null lengths");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (fused_scan_possible(tbe, batch_size, num_keys, num_indices, pooling_mode, lengths))
+    return forward_impl(tbe, weights, indices, lengths, true, idx_is_i64, per_sample_weights,
+                        batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream);
+  // Offsets first, then the ordinary lookup.
+  const int64_t n = (int64_t)num_keys * batch_size;
+  if (!workspace) {
+    set_error("tra_tbe_forward_lengths: workspace of %lld bytes required",
+              (long long)tra_tbe_forward_lengths_workspace_bytes(num_keys, batch_size, idx_is_i64));
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int64_t off_bytes = ((n + 1) * (idx_is_i64 ? 8 : 4) + 255) / 256 * 256;
+  void* scan_ws = tra_cumsum_workspace_bytes(n) ? (void*)((uint8_t*)workspace + off_bytes) : nullptr;
+  const int rc = tra_cumsum(lengths, n, idx_is_i64, workspace, scan_ws, stream);
+  if (rc != TRA_OK) return rc;
+  return forward_impl(tbe, weights, indices, workspace, false, idx_is_i64, per_sample_weights,
+                      batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream);
 }
 
 int tra_tbe_error_count(tra_tbe_t tbe, void* stream, int64_t* count) {

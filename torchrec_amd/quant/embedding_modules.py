@@ -409,7 +409,19 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         order = self._resolve_order(_get_kjt_keys(features))
         B = features.stride()
         indices = features.values()
-        offsets = features.offsets()
+        # A KJT that was built from lengths and has not had its offsets asked
+        # for goes to a single operator as it is: the operator derives the
+        # offsets itself (inside the lookup kernel when the call is large).
+        lengths = None
+        if (
+            len(self._emb_modules) == 1
+            and features.offsets_or_none() is None
+            and features.lengths_or_none() is not None
+            and B > 0
+        ):
+            offsets, lengths = None, features.lengths()
+        else:
+            offsets = features.offsets()
         psw = features.weights() if self._is_weighted else None
         total_D = sum(self._length_per_key)
         out = torch.empty((B, total_D), dtype=self._output_dtype, device=indices.device)
@@ -419,6 +431,7 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
             emb_op.forward(  # type: ignore[operator]
                 indices=indices,
                 offsets=offsets,
+                lengths=lengths,
                 per_sample_weights=psw,
                 feature_positions=order[f0 : f0 + n_feat],
                 batch_size=B,

@@ -131,6 +131,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             total = round_up(total + r * rb, _TABLE_ALIGNMENT)
         self.weights_size: int = total
         self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
+        self._workspace: Optional[Tensor] = None  # scratch of forward(offsets=None, lengths=...)
         self._weights_initialized = False
         self.weight_initialized = False
         self.register_buffer("weights_dev", torch.empty(0, dtype=torch.uint8, device=device), persistent=False)
@@ -255,6 +256,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         batch_size: Optional[int] = None,
         out: Optional[Tensor] = None,
         out_col: int = 0,
+        lengths: Optional[Tensor] = None,
     ) -> Tensor:
         """Pooled: ``[B, total_D]``; ``PoolingMode.NONE``: ``[indices.numel(), D]``.
 
@@ -265,7 +267,10 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         ``offsets[feature_positions[f] * B + b]`` with ``B = batch_size``;
         ``out`` / ``out_col`` make the operator write into columns
         ``out_col ..`` of a caller-owned ``[B, >= out_col + total_D]`` tensor
-        (``[L, D]`` for PoolingMode.NONE).
+        (``[L, D]`` for PoolingMode.NONE).  With ``offsets=None`` and
+        ``lengths`` (the KJT's ``[K * B]`` lengths, ``batch_size`` required) the
+        operator derives the offsets itself, inside the lookup kernel when the
+        call is large enough for that to pay.
         """
         dev = self.current_device
         if dev.type != "cuda":
@@ -276,13 +281,20 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         if not self._weights_initialized:
             raise _lib.TorchrecAmdError("weights are not initialized (call initialize_weights())")
         _lib.require_gpu(indices, "indices")
-        _lib.require_gpu(offsets, "offsets")
         if indices.dtype not in (torch.int32, torch.int64):
             raise TypeError(f"indices must be int32 or int64, got {indices.dtype}")
-        if offsets.dtype != indices.dtype:
-            offsets = offsets.to(indices.dtype)
         indices = indices.contiguous()
-        offsets = offsets.contiguous()
+        if offsets is None:
+            assert lengths is not None and batch_size is not None, "offsets=None needs lengths and batch_size"
+            _lib.require_gpu(lengths, "lengths")
+            if lengths.dtype != indices.dtype:
+                lengths = lengths.to(indices.dtype)
+            lengths = lengths.contiguous().view(-1)
+        else:
+            _lib.require_gpu(offsets, "offsets")
+            if offsets.dtype != indices.dtype:
+                offsets = offsets.to(indices.dtype)
+            offsets = offsets.contiguous()
         F = len(self.feature_table_map)
         positions: Optional[Tuple[int, ...]] = None
         if feature_positions is not None:
@@ -295,7 +307,12 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             batch_size = (offsets.numel() - 1) // F
         B = int(batch_size)
         n_keys = (max(positions) + 1) if positions else F
-        assert offsets.numel() >= n_keys * B + 1, "offsets shorter than the features it must cover"
+        if offsets is None:
+            assert B == 0 or lengths.numel() % B == 0, "lengths must have K * B entries"
+            k_total = lengths.numel() // B if B else n_keys
+            assert k_total >= n_keys, "lengths shorter than the features it must cover"
+        else:
+            assert offsets.numel() >= n_keys * B + 1, "offsets shorter than the features it must cover"
         L = indices.numel()
         out_dtype = torch.float16 if self.output_dtype == _lib.FP16 else torch.float32
         nobag = self.pooling_mode == PoolingMode.NONE
@@ -317,13 +334,26 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 assert out.shape[0] >= B and out.shape[1] >= out_col + self.total_D
         out_stride = out.stride(0)
         out_ptr = ctypes.c_void_p(out.data_ptr() + out_col * out.element_size())
-        _lib.check(
-            _lib.lib().tra_tbe_forward(
-                self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices), _lib.ptr(offsets),
-                int(indices.dtype == torch.int64), _lib.ptr(psw), B, L, int(self.pooling_mode),
-                self.output_dtype, out_ptr, out_stride, _lib.current_stream(dev),
+        i64 = int(indices.dtype == torch.int64)
+        if offsets is None:
+            ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
+            if self._workspace is None or self._workspace.numel() < ws_bytes or self._workspace.device != dev:
+                self._workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+            _lib.check(
+                _lib.lib().tra_tbe_forward_lengths(
+                    self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices), _lib.ptr(lengths),
+                    i64, _lib.ptr(psw), B, k_total, L, int(self.pooling_mode),
+                    self.output_dtype, out_ptr, out_stride, _lib.ptr(self._workspace), _lib.current_stream(dev),
+                )
             )
-        )
+        else:
+            _lib.check(
+                _lib.lib().tra_tbe_forward(
+                    self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices), _lib.ptr(offsets),
+                    i64, _lib.ptr(psw), B, L, int(self.pooling_mode),
+                    self.output_dtype, out_ptr, out_stride, _lib.current_stream(dev),
+                )
+            )
         if os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1":
             bad = self.out_of_range_count()
             if bad:
