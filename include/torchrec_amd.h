@@ -133,12 +133,16 @@ int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indi
 
 /* Which kernels a tra_tbe_forward with these sizes launches, one entry per
  * launch, "; "-separated, e.g. "tbe_pooled_cu_kernel dtype=int4 lane_bytes=8
- * slices=26".  For profiling: the names are the ones a kernel trace shows.
+ * slices=26".  lengths_num_keys > 0 asks about tra_tbe_forward_lengths with
+ * that many keys instead (entries then end in " from_lengths" when the kernel
+ * derives the offsets itself, else the scan kernels come first).  For
+ * profiling: the names are the ones a kernel trace shows.
  * No counterpart in the reference: fbgemm_gpu picks its kernel inside the
  * TBE module's forward (called at torchrec/quant/embedding_modules.py:547-557)
  * and does not report it. */
 int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
-                        int32_t pooling_mode, char* buf, int32_t buf_len);
+                        int32_t pooling_mode, int32_t lengths_num_keys, char* buf,
+                        int32_t buf_len);
 
 /* Number of out-of-range ids seen by forwards on this plan since the last
  * call (synchronizes the stream; resets the counter).  Stands in for

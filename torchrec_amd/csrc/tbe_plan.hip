@@ -269,29 +269,6 @@ static bool use_window_kernel(const tra_tbe* tbe, const Tuning& tune, bool nobag
   return balanced;
 }
 
-int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
-                        int32_t pooling_mode, char* buf, int32_t buf_len) {
-  if (!tbe || !buf || buf_len <= 0) {
-    set_error("tra_tbe_launch_info: null argument");
-    return TRA_ERR_INVALID_ARGUMENT;
-  }
-  const bool nobag = pooling_mode == TRA_POOL_NONE;
-  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
-  const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
-  static const char* const kDtypeName[] = {"fp32", "fp16", "int8", "int4", "int2"};
-  std::string text;
-  for (const LaunchClass& cls : tbe->classes) {
-    char line[160];
-    snprintf(line, sizeof(line), "%s%s dtype=%s lane_bytes=%d slices=%d",
-             text.empty() ? "" : "; ",
-             nobag ? "tbe_nobag_kernel" : (balanced ? "tbe_pooled_cu_kernel" : "tbe_pooled_kernel"),
-             kDtypeName[cls.dtype], cls.cb, (int)cls.feats.size());
-    text += line;
-  }
-  snprintf(buf, (size_t)buf_len, "%s", text.c_str());
-  return TRA_OK;
-}
-
 // Largest number of features one window of the from-lengths kernel may span.
 constexpr int kMaxWindowFeatures = 32;
 
@@ -312,6 +289,35 @@ static bool fused_scan_possible(const tra_tbe* tbe, int32_t batch_size, int32_t 
   // about 7 us once.  Take whichever is less.
   const int64_t n = (int64_t)num_keys * batch_size;
   return (int64_t)tbe->classes.size() * (13 + n / 4000) < 70;
+}
+
+int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
+                        int32_t pooling_mode, int32_t lengths_num_keys, char* buf,
+                        int32_t buf_len) {
+  if (!tbe || !buf || buf_len <= 0) {
+    set_error("tra_tbe_launch_info: null argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const bool nobag = pooling_mode == TRA_POOL_NONE;
+  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
+  const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
+  // lengths entry point: same decision as tra_tbe_forward_lengths (aligned lengths assumed)
+  const bool fused = lengths_num_keys > 0 &&
+                     fused_scan_possible(tbe, batch_size, lengths_num_keys, num_indices, pooling_mode,
+                                         (const void*)16);
+  static const char* const kDtypeName[] = {"fp32", "fp16", "int8", "int4", "int2"};
+  std::string text;
+  for (const LaunchClass& cls : tbe->classes) {
+    char line[160];
+    snprintf(line, sizeof(line), "%s%s dtype=%s lane_bytes=%d slices=%d%s",
+             text.empty() ? "" : "; ",
+             nobag ? "tbe_nobag_kernel" : (balanced ? "tbe_pooled_cu_kernel" : "tbe_pooled_kernel"),
+             kDtypeName[cls.dtype], cls.cb, (int)cls.feats.size(), fused ? " from_lengths" : "");
+    text += line;
+  }
+  if (lengths_num_keys > 0 && !fused) text = "scan_small_kernel or tile_sums_kernel + scan_tiles_kernel; " + text;
+  snprintf(buf, (size_t)buf_len, "%s", text.c_str());
+  return TRA_OK;
 }
 
 static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
