@@ -15,6 +15,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
 #include <vector>
 
 #include "tra_common.h"
@@ -53,6 +54,7 @@ struct LookupArgs {
   int32_t vec_store;  // 1: every lane's output slice is 16-byte aligned
   int32_t out_fp16;
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
+  int32_t deal;         // balanced pooled kernel: how rounds are dealt to waves (tuning)
   int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
 #ifdef TRA_INSTRUMENT
   unsigned long long* ts;  // [waves][8] wall-clock stamps
@@ -191,15 +193,33 @@ struct RowBuf {
   int valid;  // 1: accumulate; 0: skip
 };
 
+// Everything a lane needs to walk rows of its feature's table.
+struct RowWalk {
+  const uint8_t* lane_base;  // table + this lane's chunk offset inside a row
+  int64_t rows;
+  uint32_t rows32;     // min(rows, 2^31): bound for int32 ids
+  uint32_t row_bytes;
+  int chunk_off;
+  bool count_errors;
+  __device__ __forceinline__ void set_rows(int64_t r, int32_t rb) {
+    rows = r;
+    rows32 = r < (int64_t(1) << 31) ? (uint32_t)r : 0x80000000u;
+    row_bytes = (uint32_t)rb;
+  }
+};
+
 // Id of position j, or -1 (= skip) when the position is outside the bag.  The
 // load itself is unconditional (position clamped into the ids array) and the
 // result is selected afterwards: a load under a lane predicate would be
 // followed by a full wait at the re-convergence point and serialize the ids.
 template <typename IdxT>
-__device__ __forceinline__ int64_t fetch_id(const LookupArgs& a, bool in_range, int64_t j) {
-  const int64_t jc = j < a.num_indices ? j : a.num_indices - 1;
-  const int64_t id = load_index<IdxT>(a.indices, jc);
-  return in_range ? id : (int64_t)-1;
+__device__ __forceinline__ IdxT fetch_id(const LookupArgs& a, bool in_range, IdxT j, IdxT last) {
+  // Ids and positions stay in the width of the index type: with int32 ids the
+  // whole address computation is 32-bit (plus one 64-bit add to the base).
+  using UIdxT = typename std::make_unsigned<IdxT>::type;
+  const IdxT jc = (UIdxT)j < (UIdxT)last ? j : last;  // also catches a wrapped position
+  const IdxT id = reinterpret_cast<const IdxT*>(a.indices)[jc];
+  return in_range ? id : (IdxT)-1;
 }
 
 // Issue the loads of one row chunk (header dword, CB payload bytes, weight).
@@ -207,13 +227,24 @@ __device__ __forceinline__ int64_t fetch_id(const LookupArgs& a, bool in_range, 
 // its bag, or a bad id) is redirected to row 0 and flagged invalid; consume_row
 // then multiplies it away exactly.  Returns 1 for a bad id (out of range and
 // not -1).
-template <int DTYPE, int CB, bool WEIGHTED>
-__device__ __forceinline__ int fetch_row(RowBuf<CB>& r, int64_t id, int64_t j,
-                                          const LookupArgs& a, const uint8_t* lane_base,
-                                          int64_t rows, int64_t row_bytes, int chunk_off) {
-  const bool valid = (uint64_t)id < (uint64_t)rows;
-  const int64_t idc = valid ? id : 0;
-  const uint8_t* chunk = lane_base + idc * row_bytes;  // lane_base = table + chunk_off
+template <int DTYPE, int CB, bool WEIGHTED, typename IdxT>
+__device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT last,
+                                          const LookupArgs& a, const RowWalk& w) {
+  const uint8_t* lane_base = w.lane_base;  // table + this lane's chunk offset
+  const int chunk_off = w.chunk_off;
+  bool valid;
+  const uint8_t* chunk;
+  if constexpr (sizeof(IdxT) == 4) {
+    // One unsigned compare covers negative ids; the row address is a single
+    // 32 x 32 + 64 bit multiply-add.
+    valid = (uint32_t)id < w.rows32;
+    const uint32_t idc = valid ? (uint32_t)id : 0u;
+    chunk = lane_base + (uint64_t)idc * (uint64_t)w.row_bytes;
+  } else {
+    valid = (uint64_t)id < (uint64_t)w.rows;
+    const int64_t idc = valid ? (int64_t)id : 0;
+    chunk = lane_base + idc * (int64_t)w.row_bytes;
+  }
 #ifdef TRA_EXP_NO_ROW_LOADS
   r.hdr = 0x3c003c00u;
 #pragma unroll
@@ -226,13 +257,14 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, int64_t id, int64_t j,
   r.d = load_chunk<CB>(chunk);
 #endif
   if constexpr (WEIGHTED) {
-    const int64_t jc = j < a.num_indices ? j : a.num_indices - 1;
+    using UIdxT = typename std::make_unsigned<IdxT>::type;
+    const IdxT jc = (UIdxT)j < (UIdxT)last ? j : last;
     r.w = a.psw[jc];
   } else {
     r.w = 1.0f;
   }
   r.valid = valid;
-  return (!valid && id != -1) ? 1 : 0;
+  return (!valid && id != (IdxT)-1) ? 1 : 0;
 }
 
 // Accumulate one fetched row chunk.  An invalid row contributes fmaf(+0, q,
@@ -249,14 +281,18 @@ __device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r) {
   constexpr int EPD = 32 / Traits<DTYPE>::kBits;  // elements per dword
   float s, b;
   if constexpr (Traits<DTYPE>::kHeader != 0) {
-    s = half_bits_to_float(r.hdr & 0xffffu);
-    b = half_bits_to_float(r.hdr >> 16);
     if constexpr (WEIGHTED) {
-      s = r.w * s;
-      b = r.w * b;
+      // The weight of a skipped slot is whatever lies at the clamped
+      // position, possibly inf / nan: select after the products.
+      s = r.w * half_bits_to_float(r.hdr & 0xffffu);
+      b = r.w * half_bits_to_float(r.hdr >> 16);
+      s = r.valid ? s : 0.0f;
+      b = r.valid ? b : 0.0f;
+    } else {
+      const uint32_t hdr = r.valid ? r.hdr : 0u;  // scale = bias = +0
+      s = half_bits_to_float(hdr & 0xffffu);
+      b = half_bits_to_float(hdr >> 16);
     }
-    s = r.valid ? s : 0.0f;
-    b = r.valid ? b : 0.0f;
 #pragma unroll
     for (int i = 0; i < CB / 4; ++i)
       accumulate_dword<DTYPE, WEIGHTED>(acc + i * EPD, r.d.v[i], s, b);
@@ -347,14 +383,6 @@ __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lp
 #endif
 
 // ---- pooled lookup ----------------------------------------------------------
-// Everything a lane needs to walk rows of its feature's table.
-struct RowWalk {
-  const uint8_t* lane_base;  // table + this lane's chunk offset inside a row
-  int64_t rows;
-  int64_t row_bytes;
-  int chunk_off;
-  bool count_errors;
-};
 
 // Pool one bag per lane group: ids [start, start + len), in order, into acc.
 // max_len is the longest bag among the wave's lane groups (wave-uniform trip
@@ -363,43 +391,42 @@ struct RowWalk {
 // load is waited for in the batch that issued it.
 template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, int NE>
 __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
-                                         const RowWalk& w, int64_t start, int len,
+                                         const RowWalk& w, int64_t start64, int len,
                                          int max_len_any_lane) {
   // Wave-uniform by construction; telling the compiler keeps the loop control
   // on the scalar unit and the loads free of lane-mask bookkeeping.
   const int max_len = __builtin_amdgcn_readfirstlane(max_len_any_lane);
-  int64_t idA[U], idB[U];
+  const IdxT start = (IdxT)start64;
+  const IdxT last = (IdxT)(a.num_indices - 1);
+  IdxT idA[U], idB[U];
   RowBuf<CB> bufA[U], bufB[U];
   int bad = 0;
   // Row slots at or beyond max_len belong to no lane group: the (wave-uniform)
   // tests below skip their loads and their arithmetic altogether.
 #pragma unroll
-  for (int u = 0; u < U; ++u) idA[u] = fetch_id<IdxT>(a, u < len, start + u);
+  for (int u = 0; u < U; ++u) idA[u] = fetch_id<IdxT>(a, u < len, start + u, last);
 #pragma unroll
-  for (int u = 0; u < U; ++u) idB[u] = fetch_id<IdxT>(a, U + u < len, start + U + u);
+  for (int u = 0; u < U; ++u) idB[u] = fetch_id<IdxT>(a, U + u < len, start + U + u, last);
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    bad += fetch_row<DTYPE, CB, WEIGHTED>(bufA[u], idA[u], start + u, a, w.lane_base, w.rows,
-                                          w.row_bytes, w.chunk_off);
+    bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], idA[u], start + u, last, a, w);
   for (int it = 0; it < max_len; it += 2 * U) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      idA[u] = fetch_id<IdxT>(a, it + 2 * U + u < len, start + it + 2 * U + u);
+      idA[u] = fetch_id<IdxT>(a, it + 2 * U + u < len, start + it + 2 * U + u, last);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      bad += fetch_row<DTYPE, CB, WEIGHTED>(bufB[u], idB[u], start + it + U + u, a, w.lane_base,
-                                            w.rows, w.row_bytes, w.chunk_off);
+      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], idB[u], start + it + U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (it + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufA[u]);
     if (it + U >= max_len) break;
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      idB[u] = fetch_id<IdxT>(a, it + 3 * U + u < len, start + it + 3 * U + u);
+      idB[u] = fetch_id<IdxT>(a, it + 3 * U + u < len, start + it + 3 * U + u, last);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      bad += fetch_row<DTYPE, CB, WEIGHTED>(bufA[u], idA[u], start + it + 2 * U + u, a,
-                                            w.lane_base, w.rows, w.row_bytes, w.chunk_off);
+      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], idA[u], start + it + 2 * U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (it + U + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
@@ -449,8 +476,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
   RowWalk w;
   w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
   w.lane_base = a.weights + d.table_offset + w.chunk_off;
-  w.rows = d.rows;
-  w.row_bytes = d.row_bytes;
+  w.set_rows(d.rows, d.row_bytes);
   w.count_errors = c == 0 && d.payload_off == 0;
 
   float acc[NE];
@@ -483,6 +509,7 @@ constexpr int kMaxWindow = 2048;
 constexpr int kBagBits = 20;  // window entry = (feature index in sub-class << 20) | sample
 
 constexpr int kLenBins = 256;
+constexpr int kMaxWinFeat = 32;  // feature descriptors a window keeps in LDS
 
 // Sort key of a bag length: exact below 192, then steps of 64, then one bin.
 __device__ __forceinline__ int length_bin(int len) {
@@ -559,6 +586,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   __shared__ uint16_t s_order[kMaxWindow];
   __shared__ uint16_t s_slot[kMaxWindow];
   __shared__ int s_hist[kLenBins];
+  __shared__ FeatureDesc s_desc[kMaxWinFeat];
 
   TRA_STAMP(0);
   // Block -> (sub-class, window).  Consecutive windows go to the same XCD
@@ -584,6 +612,12 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     front_part = prefix_partial<IdxT>(reinterpret_cast<const IdxT*>(a.offsets),
                                       (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B), blk);
 
+  // Descriptors of the features this window touches, kept in LDS so that a
+  // round does not start with two dependent global loads.
+  {
+    const int nfeat = min((q0 + nb - 1) / a.B - fi_lo + 1, kMaxWinFeat);
+    if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = a.descs[a.feats[sc.first + fi_lo + threadIdx.x]];
+  }
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < nb; i += kCuThreads) {
@@ -707,14 +741,22 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
 
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int wave = threadIdx.x / kWaveSize;
-  const int simd = wave & 3;
   const int lpr = sc.lpr;
   const int gpw = kWaveSize / lpr;
   const int g = lane / lpr;
   const int c = lane - g * lpr;
   const int rounds = (nb + gpw - 1) / gpw;
-  for (int slot = wave >> 2; slot * 4 < rounds; slot += kCuWaves / 4) {
-    const int r = slot * 4 + ((slot & 1) ? 3 - simd : simd);
+  // Rounds are ordered longest first.  They are dealt to the 16 waves in
+  // passes that alternate direction (0..15, 15..0, ...), so the wave that got
+  // the longest round of one pass gets the shortest of the next.
+  for (int pass = 0; pass * kCuWaves < rounds; ++pass) {
+    int r;
+    if (a.deal == 0) {
+      const int slot_ = pass * 4 + (wave >> 2);
+      r = slot_ * 4 + ((slot_ & 1) ? 3 - (wave & 3) : (wave & 3));
+    } else {
+      r = pass * kCuWaves + ((pass & 1) ? kCuWaves - 1 - wave : wave);
+    }
     if (r >= rounds) continue;
     const int pos = r * gpw + g;
     const bool active = g < gpw && pos < nb;
@@ -722,7 +764,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     const uint32_t ent = s_ent[i];
     const int fi = (int)(ent >> kBagBits);
     const int b = (int)(ent & ((1u << kBagBits) - 1));
-    const FeatureDesc d = a.descs[a.feats[sc.first + fi]];
+    const FeatureDesc d = fi - fi_lo < kMaxWinFeat ? s_desc[fi - fi_lo] : a.descs[a.feats[sc.first + fi]];
     const int64_t start = s_start[i];
     const int len = active ? s_len[i] : 0;
     const int max_len = s_len[s_order[r * gpw]];  // the round's first bag is its longest
@@ -730,8 +772,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     RowWalk w;
     w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
     w.lane_base = a.weights + d.table_offset + w.chunk_off;
-    w.rows = d.rows;
-    w.row_bytes = d.row_bytes;
+    w.set_rows(d.rows, d.row_bytes);
     w.count_errors = c == 0 && d.payload_off == 0;
 
     float acc[NE];
@@ -774,15 +815,17 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
     if (i < a.n_sub && (int)blockIdx.x >= a.sub[i].tile_start) s = i;
   const int64_t stride = (int64_t)a.sub[s].tiles_per_feat * rows_per_block;
 
-  const int chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
-  const uint8_t* lane_base = a.weights + d.table_offset + chunk_off;
-  const bool count_errors = c == 0 && d.payload_off == 0;
+  RowWalk w;
+  w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
+  w.lane_base = a.weights + d.table_offset + w.chunk_off;
+  w.set_rows(d.rows, d.row_bytes);
+  w.count_errors = c == 0 && d.payload_off == 0;
   for (int64_t j = first + (int64_t)tile * rows_per_block + wave * gpw + g; j < last;
        j += stride) {
     RowBuf<CB> r;
-    const int bad = fetch_row<DTYPE, CB, false>(r, load_index<IdxT>(a.indices, j), j, a, lane_base,
-                                                 d.rows, d.row_bytes, chunk_off);
-    if (bad && count_errors) atomicAdd(a.err_count, 1ull);
+    const IdxT id = reinterpret_cast<const IdxT*>(a.indices)[j];
+    const int bad = fetch_row<DTYPE, CB, false, IdxT>(r, id, (IdxT)j, (IdxT)(a.num_indices - 1), a, w);
+    if (bad && w.count_errors) atomicAdd(a.err_count, 1ull);
     float acc[NE];
 #pragma unroll
     for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
