@@ -218,6 +218,26 @@ int tra_quantize_rows(const float* in, int64_t rows, int32_t dim, int32_t bits,
 int tra_quantize_rows_sbhalf(const float* in, int64_t rows, int32_t dim,
                              int32_t bits, uint8_t* out, void* stream);
 
+/* Positions inside bags ---------------------------------------------------- */
+/* out[j] = j - offsets[bag(j)] for j < range_size; offsets has num_bags
+ * entries (bag i ends where bag i+1 starts, the last at range_size), out the
+ * same integer type.  Replaces torch.ops.fbgemm.offsets_range
+ * (torchrec/modules/feature_processor_.py:82-84, 193-207). */
+int tra_offsets_range(const void* offsets, int64_t num_bags, int32_t is_i64,
+                      int64_t range_size, void* out, void* stream);
+/* Per-id position weights of a KJT: for key k with key_len[k] > 0,
+ * out[j] = table[key_start[k] + (j - start of j's bag)]; 1.0f for keys with
+ * key_len[k] <= 0.  offsets: device [num_keys*batch_size + 1]; key_start,
+ * key_len: device int32 [num_keys]; table: device fp32 (all keys' position
+ * weights back to back).  One launch for what the reference does with
+ * offsets_range + split by length_per_key (a host sync) + gather + cat
+ * (torchrec/modules/feature_processor_.py:140-155, 193-220).  A position at
+ * or beyond key_len[k] takes the last entry (the reference's gather raises). */
+int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys,
+                         int32_t batch_size, const int32_t* key_start,
+                         const int32_t* key_len, const float* table, float* out,
+                         void* stream);
+
 /* Measurement ------------------------------------------------------------- */
 /* Streaming device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte
  * aligned pointers) by a kernel named tra_copy_kernel.  A copy of known size

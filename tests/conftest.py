@@ -10,6 +10,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # quantize_dynamic (the swap mechanism the reference uses too) announces its deprecation on every call
+    config.addinivalue_line("filterwarnings", "ignore:torch.ao.quantization is deprecated:DeprecationWarning")
 
 
 def pytest_collection_modifyitems(config, items):

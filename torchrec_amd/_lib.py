@@ -37,6 +37,8 @@ EXPORTED_SYMBOLS = [
     "tra_bucketize_scatter",
     "tra_quantize_rows",
     "tra_quantize_rows_sbhalf",
+    "tra_offsets_range",
+    "tra_position_weights",
     "tra_copy_bytes",
 ]
 
@@ -95,6 +97,8 @@ def lib() -> ctypes.CDLL:
         l.tra_bucketize_scatter.argtypes = [vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp]
         l.tra_quantize_rows.argtypes = [vp, i64, i32, i32, vp, i32, vp]
         l.tra_quantize_rows_sbhalf.argtypes = [vp, i64, i32, i32, vp, vp]
+        l.tra_offsets_range.argtypes = [vp, i64, i32, i64, vp, vp]
+        l.tra_position_weights.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp]
         l.tra_copy_bytes.argtypes = [vp, vp, i64, vp]
         _lib = l
     return _lib

@@ -313,6 +313,40 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* in, int
   }
 }
 
+// ---- positions inside bags ---------------------------------------------------
+// One thread per bag: range[j] = j - start(bag) for the bag's ids.
+template <typename T>
+__global__ void offsets_range_kernel(const void* offsets, int64_t n, int64_t range_size, void* out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t s = ld<T>(offsets, i);
+  const int64_t e = i + 1 < n ? ld<T>(offsets, i + 1) : range_size;
+  for (int64_t j = s; j < e && j < range_size; ++j) st<T>(out, j, j - s);
+}
+
+// One thread per bag of key k: weight[j] = table[key_start[k] + (j - start)],
+// 1.0 for keys without a table.  Positions at or beyond the key's table length
+// take the last entry.
+template <typename T>
+__global__ void position_weights_kernel(const void* offsets, int32_t B, int64_t n,
+                                        const int32_t* key_start, const int32_t* key_len,
+                                        const float* table, float* out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int k = (int)(i / B);
+  const int64_t s = ld<T>(offsets, i), e = ld<T>(offsets, i + 1);
+  const int len = key_len[k];
+  if (len <= 0) {
+    for (int64_t j = s; j < e; ++j) out[j] = 1.0f;
+    return;
+  }
+  const float* t = table + key_start[k];
+  for (int64_t j = s; j < e; ++j) {
+    const int64_t pos = j - s;
+    out[j] = t[pos < len ? pos : len - 1];
+  }
+}
+
 // Plain streaming copy, 16 bytes per lane per step.
 __global__ __launch_bounds__(256) void tra_copy_kernel(const uint4* __restrict__ src,
                                                         uint4* __restrict__ dst, int64_t n16) {
@@ -560,6 +594,50 @@ int tra_quantize_rows_sbhalf(const float* in, int64_t rows, int32_t dim, int32_t
                              uint8_t* out, void* stream) {
   const int64_t rb = bits > 0 && bits <= 8 ? (int64_t)dim * bits / 8 + 4 : 0;
   return quantize_impl(in, rows, dim, bits, out, rb, 0, (hipStream_t)stream);
+}
+
+int tra_offsets_range(const void* offsets, int64_t num_bags, int32_t is_i64, int64_t range_size,
+                      void* out, void* stream) {
+  if (num_bags < 0 || range_size < 0) {
+    set_error("tra_offsets_range: negative size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (num_bags == 0 || range_size == 0) return TRA_OK;
+  if (!offsets || !out) {
+    set_error("tra_offsets_range: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  dim3 g((unsigned)((num_bags + 127) / 128)), b(128);
+  if (is_i64)
+    hipLaunchKernelGGL(offsets_range_kernel<int64_t>, g, b, 0, (hipStream_t)stream, offsets, num_bags,
+                       range_size, out);
+  else
+    hipLaunchKernelGGL(offsets_range_kernel<int32_t>, g, b, 0, (hipStream_t)stream, offsets, num_bags,
+                       range_size, out);
+  return check_launch("tra_offsets_range");
+}
+
+int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys, int32_t batch_size,
+                         const int32_t* key_start, const int32_t* key_len, const float* table,
+                         float* out, void* stream) {
+  if (num_keys < 0 || batch_size < 0) {
+    set_error("tra_position_weights: negative size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int64_t n = (int64_t)num_keys * batch_size;
+  if (n == 0) return TRA_OK;
+  if (!offsets || !key_start || !key_len) {
+    set_error("tra_position_weights: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  dim3 g((unsigned)((n + 127) / 128)), b(128);
+  if (is_i64)
+    hipLaunchKernelGGL(position_weights_kernel<int64_t>, g, b, 0, (hipStream_t)stream, offsets,
+                       batch_size, n, key_start, key_len, table, out);
+  else
+    hipLaunchKernelGGL(position_weights_kernel<int32_t>, g, b, 0, (hipStream_t)stream, offsets,
+                       batch_size, n, key_start, key_len, table, out);
+  return check_launch("tra_position_weights");
 }
 
 int tra_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream) {

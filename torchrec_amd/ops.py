@@ -229,3 +229,52 @@ def FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(weight: torch.Tensor, bit_rate:
         )
         out_host[r0 : r0 + n].copy_(out)
     return out_host
+
+
+def offsets_range(offsets: torch.Tensor, range_size: int) -> torch.Tensor:
+    """[num_bags] bag starts -> [range_size] position of every element inside its bag
+    (torch.ops.fbgemm.offsets_range; torchrec/modules/feature_processor_.py:82-84)."""
+    _check_int(offsets, "offsets")
+    offsets = offsets.reshape(-1).contiguous()
+    n = offsets.numel()
+    if offsets.device.type != "cuda":
+        if n == 0 or range_size == 0:
+            return offsets.new_zeros(range_size)
+        ends = torch.cat([offsets[1:], offsets.new_tensor([range_size])])
+        lengths = (ends - offsets).clamp(min=0)
+        starts = torch.repeat_interleave(offsets, lengths)
+        return torch.arange(range_size, dtype=offsets.dtype)[: starts.numel()] - starts
+    out = torch.zeros(range_size, dtype=offsets.dtype, device=offsets.device)
+    _lib.check(
+        _lib.lib().tra_offsets_range(
+            _lib.ptr(offsets), n, int(offsets.dtype == torch.int64), range_size, _lib.ptr(out),
+            _lib.current_stream(offsets.device),
+        )
+    )
+    return out
+
+
+def position_weights(
+    offsets: torch.Tensor,
+    num_keys: int,
+    batch_size: int,
+    key_start: torch.Tensor,
+    key_len: torch.Tensor,
+    table: torch.Tensor,
+    num_values: int,
+) -> torch.Tensor:
+    """Per-id weights ``table[key_start[k] + position in bag]`` (1.0 where ``key_len[k] <= 0``)
+    for a feature-major KJT with ``offsets`` of ``num_keys * batch_size + 1`` entries."""
+    _check_int(offsets, "offsets")
+    _lib.require_gpu(offsets, "offsets")
+    offsets = offsets.contiguous()
+    assert offsets.numel() >= num_keys * batch_size + 1
+    assert key_start.dtype == torch.int32 and key_len.dtype == torch.int32 and table.dtype == torch.float32
+    out = torch.empty(num_values, dtype=torch.float32, device=offsets.device)
+    _lib.check(
+        _lib.lib().tra_position_weights(
+            _lib.ptr(offsets), int(offsets.dtype == torch.int64), num_keys, batch_size, _lib.ptr(key_start),
+            _lib.ptr(key_len), _lib.ptr(table.contiguous()), _lib.ptr(out), _lib.current_stream(offsets.device),
+        )
+    )
+    return out

@@ -49,6 +49,10 @@ from torchrec_amd.modules.embedding_modules import (
     EmbeddingCollectionInterface,
     get_embedding_names_by_table,
 )
+from torchrec_amd.modules.feature_processor_ import FeatureProcessorsCollection
+from torchrec_amd.modules.fp_embedding_modules import (
+    FeatureProcessedEmbeddingBagCollection as OriginalFeatureProcessedEmbeddingBagCollection,
+)
 from torchrec_amd.modules.utils import _get_batching_hinted_output
 from torchrec_amd.sparse.jagged_tensor import (
     ComputeKJTToJTDict,
@@ -488,6 +492,83 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
     @property
     def device(self) -> torch.device:
         return self._device
+
+
+class FeatureProcessedEmbeddingBagCollection(EmbeddingBagCollection):
+    """Quantized collection behind a feature processor
+    (torchrec/quant/embedding_modules.py:633-731): ``forward`` first lets
+    ``feature_processor`` attach per-id weights to the KJT, then runs the
+    weighted lookup."""
+
+    def __init__(
+        self,
+        tables: List[EmbeddingBagConfig],
+        is_weighted: bool,
+        device: torch.device,
+        output_dtype: torch.dtype = torch.float,
+        table_name_to_quantized_weights: Optional[Dict[str, Tuple[Tensor, Tensor]]] = None,
+        register_tbes: bool = False,
+        quant_state_dict_split_scale_bias: bool = False,
+        row_alignment: int = DEFAULT_ROW_ALIGNMENT,
+        # Optional only because it is the last positional argument; without a
+        # feature processor use EmbeddingBagCollection.
+        feature_processor: Optional[FeatureProcessorsCollection] = None,
+        cache_features_order: bool = False,
+    ) -> None:
+        super().__init__(
+            tables,
+            is_weighted,
+            device,
+            output_dtype,
+            table_name_to_quantized_weights,
+            register_tbes,
+            quant_state_dict_split_scale_bias,
+            row_alignment,
+            cache_features_order,
+        )
+        assert feature_processor is not None, "Use EmbeddingBagCollection for no feature_processor"
+        self.feature_processor: FeatureProcessorsCollection = feature_processor
+
+    def forward(self, features: KeyedJaggedTensor) -> KeyedTensor:
+        return super().forward(self.feature_processor(features))
+
+    def _get_name(self) -> str:
+        return "QuantFeatureProcessedEmbeddingBagCollection"
+
+    @classmethod
+    def from_float(  # type: ignore[override]
+        cls, module: OriginalFeatureProcessedEmbeddingBagCollection, use_precomputed_fake_quant: bool = False
+    ) -> "FeatureProcessedEmbeddingBagCollection":
+        assert hasattr(
+            module, "qconfig"
+        ), "FeatureProcessedEmbeddingBagCollection input float module must have qconfig defined"
+        ebc = module._embedding_bag_collection
+        qconfig = module.qconfig
+        pruning_dict: Dict[str, int] = getattr(
+            module, MODULE_ATTR_EMB_CONFIG_NAME_TO_NUM_ROWS_POST_PRUNING_DICT, {}
+        )
+        embedding_bag_configs = copy.deepcopy(ebc.embedding_bag_configs())
+        _update_embedding_configs(embedding_bag_configs, qconfig, pruning_dict)
+        table_name_to_quantized_weights: Dict[str, Tuple[Tensor, Tensor]] = {}
+        device = quantize_state_dict(
+            ebc,
+            table_name_to_quantized_weights,
+            {table.name: table.data_type for table in embedding_bag_configs},
+            pruning_dict,
+        )
+        feature_processor, _ = module.split()  # a per-feature dict is wrapped into a collection
+        return cls(
+            embedding_bag_configs,
+            ebc.is_weighted(),
+            device=device,
+            output_dtype=qconfig.activation().dtype,
+            table_name_to_quantized_weights=table_name_to_quantized_weights,
+            register_tbes=getattr(module, MODULE_ATTR_REGISTER_TBES_BOOL, False),
+            quant_state_dict_split_scale_bias=getattr(ebc, MODULE_ATTR_QUANT_STATE_DICT_SPLIT_SCALE_BIAS, False),
+            row_alignment=getattr(ebc, MODULE_ATTR_ROW_ALIGNMENT_INT, DEFAULT_ROW_ALIGNMENT),
+            feature_processor=feature_processor,
+            cache_features_order=getattr(module, MODULE_ATTR_CACHE_FEATURES_ORDER, False),
+        )
 
 
 # ---------------------------------------------------------------------------
