@@ -238,6 +238,17 @@ int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys,
                          const int32_t* key_len, const float* table, float* out,
                          void* stream);
 
+/* Managed-collision id remap ------------------------------------------------ */
+/* out[j] = mapping[i] if sorted_ids[i] == values[j], where i is the lower
+ * bound of values[j] among the first table_size-1 entries of sorted_ids
+ * (ascending int64; the last entry is the delimiter), else miss_id.  values
+ * and out: device [n] int32 or int64; sorted_ids, mapping: device int64
+ * [table_size].  Replaces _mch_remap (searchsorted + gather + masked writes,
+ * torchrec/modules/mc_modules.py:959-989). */
+int tra_mch_remap(const void* values, int64_t n, int32_t is_i64,
+                  const int64_t* sorted_ids, const int64_t* mapping,
+                  int64_t table_size, int64_t miss_id, void* out, void* stream);
+
 /* Measurement ------------------------------------------------------------- */
 /* Streaming device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte
  * aligned pointers) by a kernel named tra_copy_kernel.  A copy of known size

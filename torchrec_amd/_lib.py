@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = [
     "tra_quantize_rows_sbhalf",
     "tra_offsets_range",
     "tra_position_weights",
+    "tra_mch_remap",
     "tra_copy_bytes",
 ]
 
@@ -99,6 +100,7 @@ def lib() -> ctypes.CDLL:
         l.tra_quantize_rows_sbhalf.argtypes = [vp, i64, i32, i32, vp, vp]
         l.tra_offsets_range.argtypes = [vp, i64, i32, i64, vp, vp]
         l.tra_position_weights.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp]
+        l.tra_mch_remap.argtypes = [vp, i64, i32, vp, vp, i64, i64, vp, vp]
         l.tra_copy_bytes.argtypes = [vp, vp, i64, vp]
         _lib = l
     return _lib

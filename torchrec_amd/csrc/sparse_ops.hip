@@ -347,6 +347,25 @@ __global__ void position_weights_kernel(const void* offsets, int32_t B, int64_t 
   }
 }
 
+// ---- id remapping through a sorted table --------------------------------------
+// out[j] = mapping[i] when sorted_ids[i] == values[j] with i the first index in
+// [0, size-1] whose entry is >= values[j] (searched over the first size-1
+// entries; the last one is the table's delimiter), else miss_id.
+template <typename T>
+__global__ void mch_remap_kernel(const void* values, int64_t n, const int64_t* sorted_ids,
+                                 const int64_t* mapping, int64_t size, int64_t miss_id, void* out) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += stride) {
+    const int64_t v = ld<T>(values, j);
+    int64_t lo = 0, hi = size - 1;  // lower bound in [0, size - 1)
+    while (lo < hi) {
+      const int64_t mid = lo + ((hi - lo) >> 1);
+      if (sorted_ids[mid] < v) lo = mid + 1; else hi = mid;
+    }
+    st<T>(out, j, sorted_ids[lo] == v ? mapping[lo] : miss_id);
+  }
+}
+
 // Plain streaming copy, 16 bytes per lane per step.
 __global__ __launch_bounds__(256) void tra_copy_kernel(const uint4* __restrict__ src,
                                                         uint4* __restrict__ dst, int64_t n16) {
@@ -638,6 +657,28 @@ int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys, 
     hipLaunchKernelGGL(position_weights_kernel<int32_t>, g, b, 0, (hipStream_t)stream, offsets,
                        batch_size, n, key_start, key_len, table, out);
   return check_launch("tra_position_weights");
+}
+
+int tra_mch_remap(const void* values, int64_t n, int32_t is_i64, const int64_t* sorted_ids,
+                  const int64_t* mapping, int64_t table_size, int64_t miss_id, void* out,
+                  void* stream) {
+  if (n < 0 || table_size <= 0) {
+    set_error("tra_mch_remap: bad size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (n == 0) return TRA_OK;
+  if (!values || !sorted_ids || !mapping || !out) {
+    set_error("tra_mch_remap: null buffer");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const unsigned grid = (unsigned)std::min<int64_t>((n + 255) / 256, 256 * 16);
+  if (is_i64)
+    hipLaunchKernelGGL(mch_remap_kernel<int64_t>, dim3(grid), dim3(256), 0, (hipStream_t)stream, values,
+                       n, sorted_ids, mapping, table_size, miss_id, out);
+  else
+    hipLaunchKernelGGL(mch_remap_kernel<int32_t>, dim3(grid), dim3(256), 0, (hipStream_t)stream, values,
+                       n, sorted_ids, mapping, table_size, miss_id, out);
+  return check_launch("tra_mch_remap");
 }
 
 int tra_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream) {

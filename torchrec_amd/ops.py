@@ -278,3 +278,27 @@ def position_weights(
         )
     )
     return out
+
+
+def mch_remap(
+    values: torch.Tensor, sorted_ids: torch.Tensor, mapping: torch.Tensor, miss_id: int
+) -> torch.Tensor:
+    """Ids found in ``sorted_ids[:-1]`` (or equal to the last entry when nothing smaller is found)
+    become ``mapping[position]``, all others ``miss_id`` (torchrec/modules/mc_modules.py:959-989)."""
+    _check_int(values, "values")
+    assert sorted_ids.dtype == torch.int64 and mapping.dtype == torch.int64
+    assert sorted_ids.numel() == mapping.numel() and sorted_ids.numel() > 0
+    if values.device.type != "cuda":
+        idx = torch.searchsorted(sorted_ids[:-1], values.long())
+        hit = sorted_ids[idx] == values
+        return torch.where(hit, mapping[idx], torch.full_like(idx, miss_id)).to(values.dtype)
+    values = values.contiguous()
+    out = torch.empty_like(values)
+    _lib.check(
+        _lib.lib().tra_mch_remap(
+            _lib.ptr(values), values.numel(), int(values.dtype == torch.int64), _lib.ptr(sorted_ids.contiguous()),
+            _lib.ptr(mapping.contiguous()), sorted_ids.numel(), int(miss_id), _lib.ptr(out),
+            _lib.current_stream(values.device),
+        )
+    )
+    return out
