@@ -50,6 +50,7 @@ def parse_args():
     p.add_argument("--rocprof-summary", metavar="DIR", default=None,
                    help="no benchmark: summarize rocprofv3 CSV output under DIR (kernel_stats / counter_collection) "
                         "for this library's kernels and exit")
+    p.add_argument("--batch-size", type=int, default=None, help="override the workload's batch size (tuning only; result is then not the named workload)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink table rows (debug only; result is then invalid)")
     return p.parse_args()
 
@@ -135,6 +136,9 @@ def build_workload(args, dev):
         id_fn = None  # affine bijection below: a 250M-entry permutation per table is not needed
         desc = "c5: QEBC 8 tables x 250M x 128 int4 (68 B rows), B16384, L=80, Zipf(0.8), MEAN, fp16 out"
 
+    if getattr(args, "batch_size", None):
+        B = args.batch_size
+        desc += f" [batch size overridden to {B}]"
     if pooled:
         tables = [
             EmbeddingBagConfig(name=f"t{t}", embedding_dim=dims[t], num_embeddings=rows[t], feature_names=[f"f{t}"],

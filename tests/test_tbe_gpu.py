@@ -200,7 +200,7 @@ def test_properties_large():
 
 # The pooled lookup has two kernels: a static bag->wave mapping for small calls
 # and a per-CU window kernel that ranks bags by length (taken when a call has
-# at least 32768 bags and 524288 ids).  TRA_BALANCED / TRA_WINDOW are the
+# at least 10240 bags and 163840 ids).  TRA_BALANCED / TRA_WINDOW are the
 # library's tuning overrides; the tests below use them to put oracle-sized
 # inputs through the window kernel.
 

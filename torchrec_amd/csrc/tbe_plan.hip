@@ -56,8 +56,9 @@ constexpr int kNumCus = 256;
 
 static Tuning choose_tuning(int64_t bags, int64_t num_indices) {
   Tuning t;
-  // Ranking bags by length pays once every CU has several rounds to balance.
-  t.balanced = bags >= 128 * kNumCus && num_indices >= 2048 * (int64_t)kNumCus;
+  // Ranking bags by length pays once every CU gets a few dozen bags (measured
+  // crossover on 26 int4 tables: between 6.6k bags / 130k ids and 13k / 260k).
+  t.balanced = bags >= 40 * kNumCus && num_indices >= 640 * (int64_t)kNumCus;
   t.window = 0;
   t.unroll = 4;
   t.lds_bytes = 48 * 1024;  // with the static arrays > half of a CU's LDS: one block per CU
