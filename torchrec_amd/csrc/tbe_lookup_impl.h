@@ -245,17 +245,11 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
     const int64_t idc = valid ? (int64_t)id : 0;
     chunk = lane_base + idc * (int64_t)w.row_bytes;
   }
-#ifdef TRA_EXP_NO_ROW_LOADS
-  r.hdr = 0x3c003c00u;
-#pragma unroll
-  for (int i = 0; i < CB / 4; ++i) r.d.v[i] = (uint32_t)id * 2654435761u + i;
-#else
   if constexpr (Traits<DTYPE>::kHeader != 0)
     r.hdr = *reinterpret_cast<const uint32_t*>(chunk - chunk_off);
   else
     r.hdr = 0;
   r.d = load_chunk<CB>(chunk);
-#endif
   if constexpr (WEIGHTED) {
     using UIdxT = typename std::make_unsigned<IdxT>::type;
     const IdxT jc = (UIdxT)j < (UIdxT)last ? j : last;
@@ -274,10 +268,6 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
 // zeroed as well, so a stored inf / nan in row 0 cannot leak in.
 template <int DTYPE, int CB, bool WEIGHTED>
 __device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r) {
-#ifdef TRA_EXP_NO_DEQUANT
-  acc[0] += __builtin_bit_cast(float, r.d.v[0] ^ r.d.v[CB / 4 - 1] ^ r.hdr);
-  return;
-#endif
   constexpr int EPD = 32 / Traits<DTYPE>::kBits;  // elements per dword
   float s, b;
   if constexpr (Traits<DTYPE>::kHeader != 0) {
@@ -372,6 +362,9 @@ __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lp
   return true;
 }
 
+// Built with -DTRA_INSTRUMENT (never in the shipped library), every wave
+// records wall-clock stamps at the phases of the window kernel into a.ts; a
+// standalone harness that includes this header reads them back.
 #ifdef TRA_INSTRUMENT
 #define TRA_STAMP(k)                                                                      \
   do {                                                                                    \

@@ -357,6 +357,14 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     set_error("tra_tbe_forward: sequence lookup needs one embedding dim for all tables");
     return TRA_ERR_INVALID_ARGUMENT;
   }
+  {
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess || cur != tbe->device) {
+      set_error("tra_tbe_forward: plan was created on device %d, current device is %d", tbe->device,
+                cur);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+  }
   const int esz = out_dtype == TRA_FP16 ? 2 : 4;
   hipStream_t s = (hipStream_t)stream;
   const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
