@@ -121,6 +121,44 @@ def test_bucketize(F, B, W, idt, keep):
     assert np.array_equal(gw.cpu().numpy(), np.asarray(pw, dtype=np.float32))
 
 
+@pytest.mark.parametrize("is_sequence", [False, True])
+def test_bucketize_kjt(is_sequence):
+    """KJT-level wrappers: keys repeated per bucket, lengths/values of the op, and for
+    sequence features the unbucketize permute and the bucket of every input id."""
+    from torchrec_amd import KeyedJaggedTensor
+    from torchrec_amd.sparse.bucketize import bucketize_kjt_before_all2all, bucketize_kjt_inference
+
+    rng = np.random.default_rng(12)
+    keys, B, W = ["a", "b", "c"], 11, 4
+    lengths = rng.integers(0, 6, len(keys) * B).astype(np.int64)
+    block_sizes = np.asarray([7, 13, 29], dtype=np.int64)
+    hi = np.repeat(block_sizes * W, B)  # every id lands in a bucket
+    ids = np.concatenate([rng.integers(0, hi[i], lengths[i]) for i in range(len(lengths))]).astype(np.int64)
+    weights = rng.random(len(ids)).astype(np.float32)
+    kjt = KeyedJaggedTensor(keys=keys, values=torch.from_numpy(ids).to(DEV), lengths=torch.from_numpy(lengths).to(DEV),
+                            weights=torch.from_numpy(weights).to(DEV))
+    ol, oi, ow, ou = O.bucketize(lengths, ids, block_sizes, W, weights, False, return_permute=True)
+    out, perm, mapping = bucketize_kjt_inference(kjt, W, torch.from_numpy(block_sizes), is_sequence=is_sequence)
+    assert out.keys() == keys * W and out.stride() == B
+    assert out.lengths().cpu().numpy().tolist() == ol.tolist()
+    assert out.values().cpu().numpy().tolist() == oi.tolist()
+    assert np.array_equal(out.weights().cpu().numpy(), ow)
+    if is_sequence:
+        assert perm.cpu().numpy().tolist() == ou.tolist()
+        per_id_block = np.repeat(np.repeat(block_sizes, B), lengths)
+        assert mapping.cpu().numpy().tolist() == (ids // per_id_block).tolist()
+        # ids come back in input order through the permute
+        restored = out.values()[perm] + mapping * torch.from_numpy(per_id_block).to(DEV)
+        assert restored.cpu().numpy().tolist() == ids.tolist()
+    else:
+        assert perm is None and mapping is None
+    out2, perm2 = bucketize_kjt_before_all2all(kjt, W, torch.from_numpy(block_sizes), output_permute=is_sequence)
+    assert out2.keys() == keys * W and out2.values().cpu().numpy().tolist() == oi.tolist()
+    assert (perm2 is not None) == is_sequence
+    with pytest.raises(NotImplementedError):
+        bucketize_kjt_inference(kjt, W, torch.from_numpy(block_sizes), bucketize_pos=True)
+
+
 @pytest.mark.parametrize("bits", [8, 4, 2])
 def test_quantize_rows_bytes_identical(bits):
     rng = np.random.default_rng(bits)

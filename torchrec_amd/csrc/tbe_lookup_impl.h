@@ -54,7 +54,6 @@ struct LookupArgs {
   int32_t vec_store;  // 1: every lane's output slice is 16-byte aligned
   int32_t out_fp16;
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
-  int32_t deal;         // balanced pooled kernel: how rounds are dealt to waves (tuning)
   int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
 #ifdef TRA_INSTRUMENT
   unsigned long long* ts;  // [waves][8] wall-clock stamps
@@ -739,17 +738,14 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   const int g = lane / lpr;
   const int c = lane - g * lpr;
   const int rounds = (nb + gpw - 1) / gpw;
-  // Rounds are ordered longest first.  They are dealt to the 16 waves in
-  // passes that alternate direction (0..15, 15..0, ...), so the wave that got
-  // the longest round of one pass gets the shortest of the next.
+  // Rounds are ordered longest first and dealt to the waves four at a time,
+  // alternating direction over the four SIMDs.  (Dealing them in a strict
+  // snake over all 16 waves, or evening out the rounds per wave, measured
+  // slower: the waves that finish early leave the CU's memory pipeline to the
+  // ones still running.)
   for (int pass = 0; pass * kCuWaves < rounds; ++pass) {
-    int r;
-    if (a.deal == 0) {
-      const int slot_ = pass * 4 + (wave >> 2);
-      r = slot_ * 4 + ((slot_ & 1) ? 3 - (wave & 3) : (wave & 3));
-    } else {
-      r = pass * kCuWaves + ((pass & 1) ? kCuWaves - 1 - wave : wave);
-    }
+    const int slot = pass * 4 + (wave >> 2);
+    const int r = slot * 4 + ((slot & 1) ? 3 - (wave & 3) : (wave & 3));
     if (r >= rounds) continue;
     const int pos = r * gpw + g;
     const bool active = g < gpw && pos < nb;

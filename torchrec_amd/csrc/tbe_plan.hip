@@ -474,7 +474,6 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
       // XCD remap needs a grid that is a multiple of 8 (surplus blocks exit at once).
       lp.grid = (grid + 7) / 8 * 8;
       a.xcd_blocks = env_int("TRA_XCD", 1) ? lp.grid / 8 : 0;
-      a.deal = env_int("TRA_DEAL", 0);
     }
     lp.unroll = tune.unroll;
     lp.idx64 = idx_is_i64 != 0;
