@@ -112,6 +112,10 @@ def test_edge_bags():
     ids = np.zeros(0, dtype=np.int32)
     got, want = run_both(tbe, store, [0], B, ids, offsets, None, O.SUM, O.FP16)
     assert bits_equal(got, want) == 0 and not got.any()
+    # the same with an (empty) per-sample weight tensor
+    got = tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV),
+              torch.zeros(0, device=DEV)).cpu().numpy()
+    assert not got.any()
     # one bag of 5000 ids, the rest empty
     offsets = np.zeros(B + 1, dtype=np.int32)
     offsets[4:] = 5000

@@ -379,7 +379,8 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     // kernels need one readable element even when there are no ids at all.
     a.indices = num_indices > 0 ? indices : (const void*)tbe->err_dev;
     a.offsets = offsets;
-    a.psw = nobag ? nullptr : per_sample_weights;
+    // (no ids: nothing to weigh, and the weights pointer may not be readable)
+    a.psw = nobag || num_indices == 0 ? nullptr : per_sample_weights;
     a.out = out;
     a.out_stride = out_stride;
     a.err_count = tbe->err_dev;
