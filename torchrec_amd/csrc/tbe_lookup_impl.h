@@ -120,6 +120,8 @@ __device__ __forceinline__ float byte_to_float(uint32_t x) {
   return f;
 }
 
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
@@ -145,6 +147,26 @@ __device__ __forceinline__ void accumulate_dword(float* acc, uint32_t x, float s
     fma_step(acc[1], s, byte_to_float<1>(x), b);
     fma_step(acc[2], s, byte_to_float<2>(x), b);
     fma_step(acc[3], s, byte_to_float<3>(x), b);
+  } else if constexpr (DTYPE == TRA_INT4 && !WEIGHTED) {
+    // A byte 0x0q read as an FP8 (E4M3) value is exactly q * 2^-9 for q = 0..15
+    // (subnormals, then the first binade), and one instruction converts two
+    // bytes.  The scale is multiplied by 2^9 instead (exact: s is at most
+    // 65504 here), so every product is the same real number as s * q.
+    const uint32_t lo = x & 0x0f0f0f0fu;
+    const uint32_t hi = (x >> 4) & 0x0f0f0f0fu;
+    const float s9 = s * 512.0f;
+    const float2_t l01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false);
+    const float2_t l23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
+    const float2_t h01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false);
+    const float2_t h23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
+    fma_step(acc[0], s9, l01.x, b);
+    fma_step(acc[1], s9, h01.x, b);
+    fma_step(acc[2], s9, l01.y, b);
+    fma_step(acc[3], s9, h01.y, b);
+    fma_step(acc[4], s9, l23.x, b);
+    fma_step(acc[5], s9, h23.x, b);
+    fma_step(acc[6], s9, l23.y, b);
+    fma_step(acc[7], s9, h23.y, b);
   } else if constexpr (DTYPE == TRA_INT4) {
     const uint32_t lo = x & 0x0f0f0f0fu;
     const uint32_t hi = WEIGHTED ? ((x >> 4) & 0x0f0f0f0fu) : (x & 0xf0f0f0f0u);
@@ -157,6 +179,19 @@ __device__ __forceinline__ void accumulate_dword(float* acc, uint32_t x, float s
     fma_step(acc[5], sh, byte_to_float<2>(hi), b);
     fma_step(acc[6], s, byte_to_float<3>(lo), b);
     fma_step(acc[7], sh, byte_to_float<3>(hi), b);
+  } else if constexpr (DTYPE == TRA_INT2 && !WEIGHTED) {
+    // Same FP8 reading as for int4, on the four 2-bit fields of every byte.
+    const float s9 = s * 512.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t m = (x >> (2 * e)) & 0x03030303u;
+      const float2_t m01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)m, false);
+      const float2_t m23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)m, true);
+      fma_step(acc[0 + e], s9, m01.x, b);
+      fma_step(acc[4 + e], s9, m01.y, b);
+      fma_step(acc[8 + e], s9, m23.x, b);
+      fma_step(acc[12 + e], s9, m23.y, b);
+    }
   } else if constexpr (DTYPE == TRA_INT2) {
     float se = s;
 #pragma unroll
@@ -424,6 +459,69 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
       if (it + U + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
   }
   // Bad ids are counted by the lane that owns column 0.
+  if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
+}
+
+// The same pooling with the ids fetched a whole lane group at a time: lane c of
+// the group loads id number j*lpr + c of the bag (block j), and each row's id
+// is then passed to the group's lanes with a cross-lane read.  One id load per
+// lpr rows instead of one per row.  Needs lpr >= 2*U (a power of two): the
+// block after the current one, requested when the current one is entered, is
+// then at least two batches ahead, like the ids of pool_bag.
+template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, int NE>
+__device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs& a,
+                                              const RowWalk& w, int64_t start64, int len,
+                                              int max_len_any_lane, int lpr, int c,
+                                              int group_lane0) {
+  const int max_len = __builtin_amdgcn_readfirstlane(max_len_any_lane);
+  const int lpr_u = __builtin_amdgcn_readfirstlane(lpr);
+  const IdxT start = (IdxT)start64;
+  const IdxT last = (IdxT)(a.num_indices - 1);
+  auto load_block = [&](int j) -> IdxT {
+    const int r = j * lpr_u + c;
+    return fetch_id<IdxT>(a, r < len, start + (IdxT)r, last);
+  };
+  IdxT cur = load_block(0);
+  IdxT nxt = load_block(1);
+  int cur_j = 0;
+  // Id of row r (wave-uniform r inside block cur_j or cur_j + 1), or -1 past the bag's end.
+  auto id_of = [&](int r) -> IdxT {
+    const int j = r / lpr_u;
+    const int src = group_lane0 + (r - j * lpr_u);
+    const IdxT v = j == cur_j ? cur : nxt;
+    return (IdxT)__shfl(v, src, kWaveSize);
+  };
+  // Entering the block of row rb: make it the current one and request the next.
+  auto enter = [&](int rb) {
+    const int j = rb / lpr_u;
+    if (j > cur_j) {
+      cur = nxt;
+      nxt = load_block(j + 1);
+      cur_j = j;
+    }
+  };
+  RowBuf<CB> bufA[U], bufB[U];
+  int bad = 0;
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(u), start + u, last, a, w);
+  for (int it = 0; it < max_len; it += 2 * U) {
+    enter(it + U);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (it + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufA[u]);
+    if (it + U >= max_len) break;
+    enter(it + 2 * U);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (it + U + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
+  }
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
 }
 
@@ -767,7 +865,10 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     float acc[NE];
 #pragma unroll
     for (int k = 0; k < NE; ++k) acc[k] = 0.0f;
-    pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+    if (U == 4 && lpr >= 2 * U && (lpr & (lpr - 1)) == 0)
+      pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len, lpr, c, lane - c);
+    else
+      pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
     TRA_STAMP(3);
 #ifdef TRA_INSTRUMENT
     if (lane == 0) a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + wave) * 8 + 5] = (unsigned long long)max_len;
