@@ -322,10 +322,33 @@ class _FeatureOrderMixin:
 
     def _resolve_order(self, kjt_keys: List[str]) -> List[int]:
         if getattr(self, MODULE_ATTR_CACHE_FEATURES_ORDER, False):
+            # the reference's contract for this flag: the first key order seen is kept
             if self._features_order is None:
                 self._features_order = [kjt_keys.index(k) for k in self._feature_names]
             return self._features_order
-        return [kjt_keys.index(k) for k in self._feature_names]
+        # otherwise resolved per key order, remembered so that a repeated order costs one dict lookup
+        cache = self.__dict__.setdefault("_order_by_keys", {})
+        ck = tuple(kjt_keys)
+        order = cache.get(ck)
+        if order is None:
+            order = [kjt_keys.index(k) for k in self._feature_names]
+            if len(cache) < 64:
+                cache[ck] = order
+        return order
+
+    def _group_positions(self, order: List[int]) -> List[tuple]:
+        """``order`` cut into one tuple per lookup operator (cached per order object)."""
+        cache = self.__dict__.setdefault("_positions_by_order", {})
+        hit = cache.get(id(order))
+        if hit is not None and hit[0] is order:
+            return hit[1]
+        groups, f0 = [], 0
+        for n_feat in self._feature_splits:
+            groups.append(tuple(order[f0 : f0 + n_feat]))
+            f0 += n_feat
+        if len(cache) < 64:
+            cache[id(order)] = (order, groups)
+        return groups
 
 
 # ---------------------------------------------------------------------------
@@ -398,6 +421,7 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         )
         for table in ordered_tables:
             self._length_per_key.extend([table.embedding_dim] * len(table.feature_names))
+        self._total_D: int = sum(self._length_per_key)
 
         self.embedding_bags: nn.ModuleDict = nn.ModuleDict()
         for (_key, group_tables), emb_module in zip(self._key_to_tables.items(), self._emb_modules):
@@ -431,22 +455,19 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         else:
             offsets = features.offsets()
         psw = features.weights() if self._is_weighted else None
-        total_D = sum(self._length_per_key)
-        out = torch.empty((B, total_D), dtype=self._output_dtype, device=indices.device)
-        f0 = 0
+        out = torch.empty((B, self._total_D), dtype=self._output_dtype, device=indices.device)
         col = 0
-        for emb_op, n_feat in zip(self._emb_modules, self._feature_splits):
+        for emb_op, positions in zip(self._emb_modules, self._group_positions(order)):
             emb_op.forward(  # type: ignore[operator]
                 indices=indices,
                 offsets=offsets,
                 lengths=lengths,
                 per_sample_weights=psw,
-                feature_positions=order[f0 : f0 + n_feat],
+                feature_positions=positions,
                 batch_size=B,
                 out=out,
                 out_col=col,
             )
-            f0 += n_feat
             col += emb_op.total_D  # type: ignore[union-attr]
         return KeyedTensor(keys=self._embedding_names, values=out, length_per_key=self._length_per_key)
 

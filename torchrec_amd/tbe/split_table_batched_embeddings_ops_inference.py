@@ -131,6 +131,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             total = round_up(total + r * rb, _TABLE_ALIGNMENT)
         self.weights_size: int = total
         self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
+        self._identity_positions: Tuple[int, ...] = tuple(range(len(self.feature_table_map)))
         self._workspace: Optional[Tensor] = None  # scratch of forward(offsets=None, lengths=...)
         self._weights_initialized = False
         self.weight_initialized = False
@@ -298,8 +299,10 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         F = len(self.feature_table_map)
         positions: Optional[Tuple[int, ...]] = None
         if feature_positions is not None:
-            positions = tuple(int(p) for p in feature_positions)
-            if positions == tuple(range(F)):
+            positions = (
+                feature_positions if type(feature_positions) is tuple else tuple(int(p) for p in feature_positions)
+            )
+            if positions == self._identity_positions:
                 positions = None
         if batch_size is None:
             assert positions is None, "batch_size is required with feature_positions"
