@@ -432,3 +432,42 @@ def test_forward_from_lengths_at_scale():
     a = tbe(ti, torch.from_numpy(offsets).to(DEV))
     b = tbe(ti, None, lengths=torch.from_numpy(lengths).to(DEV), batch_size=B)
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_table_beyond_2_31_rows():
+    """A table with more than 2^31 rows (fp32, dim 1: 8.6 GB): int64 ids beyond 2^31 address the
+    right rows; int32 ids see every non-negative id as in range; ids >= rows are skipped and counted."""
+    rows, B = 2**31 + 1000, 4
+    free, _ = torch.cuda.mem_get_info()
+    if free < rows * 4 + (1 << 30):
+        pytest.skip("not enough free device memory for an 8.6 GB table")
+    tbe = TBE(embedding_specs=[("big", rows, 1, SparseType.FP32, EmbeddingLocation.DEVICE)],
+              pooling_mode=PoolingMode.SUM, device=DEV, output_dtype=SparseType.FP32, row_alignment=4)
+    tbe.initialize_weights()
+    w = tbe.weights_dev.view(torch.float32)
+    assert w.numel() >= rows
+    w.zero_()
+    picks = [0, 5, 2**31 - 1, 2**31, 2**31 + 7, rows - 1]
+    for k, r in enumerate(picks):
+        w[r] = float(k + 1)
+    ids = torch.tensor([picks[3], picks[4], picks[5], picks[0], rows, picks[2], picks[1], -1], dtype=torch.int64, device=DEV)
+    offsets = torch.tensor([0, 2, 5, 6, 8], dtype=torch.int64, device=DEV)
+    got = tbe(ids, offsets).cpu().view(-1).tolist()
+    assert got == [4.0 + 5.0, 6.0 + 1.0, 3.0, 2.0]
+    assert tbe.out_of_range_count() == 1
+    # window kernel, same ids (forced)
+    import os
+    os.environ["TRA_BALANCED"] = "1"
+    try:
+        got = tbe(ids, offsets).cpu().view(-1).tolist()
+    finally:
+        del os.environ["TRA_BALANCED"]
+    assert got == [4.0 + 5.0, 6.0 + 1.0, 3.0, 2.0]
+    assert tbe.out_of_range_count() == 1
+    # int32 ids: every non-negative id is a row of this table
+    ids32 = torch.tensor([2**31 - 1, 5, 0, -1], dtype=torch.int32, device=DEV)
+    off32 = torch.tensor([0, 1, 2, 3, 4], dtype=torch.int32, device=DEV)
+    assert tbe(ids32, off32).cpu().view(-1).tolist() == [3.0, 2.0, 1.0, 0.0]
+    assert tbe.out_of_range_count() == 0
+    del tbe, w
+    torch.cuda.empty_cache()
