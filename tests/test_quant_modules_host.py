@@ -142,3 +142,25 @@ def test_forward_without_gpu_fails_loudly():
         q(kjt)
     with pytest.raises(ValueError):  # missing feature
         q(KeyedJaggedTensor(keys=["g"], values=torch.tensor([1]), lengths=torch.tensor([1])))
+
+
+def test_feature_order_is_resolved_per_key_order():
+    """The module remembers the order it resolved for a key order, and resolves a
+    different key order afresh (the reference's cache_features_order flag, which
+    pins the first order seen, is honoured separately)."""
+    tables = [
+        EmbeddingBagConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1", "f3"], data_type=DataType.INT4),
+        EmbeddingBagConfig(name="t2", embedding_dim=32, num_embeddings=10, feature_names=["f2"], data_type=DataType.INT8, pooling=PoolingType.MEAN),
+    ]
+    q = QuantEBC(tables, False, CPU)
+    assert q._feature_names == ["f1", "f3", "f2"]
+    a = q._resolve_order(["f1", "f2", "f3"])
+    assert a == [0, 2, 1] and q._resolve_order(["f1", "f2", "f3"]) is a
+    assert q._group_positions(a) == [(0, 2), (1,)] and q._group_positions(a) is q._group_positions(a)
+    b = q._resolve_order(["x", "f3", "f2", "f1"])
+    assert b == [3, 1, 2] and q._group_positions(b) == [(3, 1), (2,)]
+    with pytest.raises(ValueError):
+        q._resolve_order(["f1", "f2"])  # a missing feature is a list.index error, as in the reference
+    pinned = QuantEBC(tables, False, CPU, cache_features_order=True)
+    first = pinned._resolve_order(["f3", "f2", "f1"])
+    assert first == [2, 0, 1] and pinned._resolve_order(["f1", "f2", "f3"]) is first
