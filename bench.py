@@ -525,8 +525,19 @@ def main():
     if not fused:
         launches = launch_info(0)
     alg = sum(wl["alg_bytes"][k % args.batches] for k in range(args.steps)) / args.steps
-    kernel_ms = time_launches(launch_lengths if fused else launch_offsets)
+    step_launch = launch_lengths if fused else launch_offsets
+    kernel_ms = time_launches(step_launch)
     achieved = alg / (kernel_ms * 1e-3) / 1e9
+    # spread of single launches: one event pair per launch (includes the launch gap)
+    singles = []
+    for k in range(min(args.steps, 200)):
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a0.record()
+        step_launch(k % NB)
+        a1.record()
+        singles.append((a0, a1))
+    torch.cuda.synchronize()
+    single_us = sorted(x.elapsed_time(y) * 1e3 for x, y in singles)
     offsets_entry = None
     if fused:
         ms = time_launches(launch_offsets)
@@ -586,6 +597,8 @@ def main():
             "kernel_ms": kernel_ms,
             "algorithmic_bytes_per_launch": alg,
             "kernel_lookups_per_s": (sum(lookups) / NB) / (kernel_ms * 1e-3),
+            "single_launch_us_p50": single_us[len(single_us) // 2],
+            "single_launch_us_p90": single_us[int(len(single_us) * 0.9)],
             "offsets_entry": offsets_entry,
         },
     }
