@@ -11,49 +11,41 @@ from torchrec_amd.modules.embedding_modules import EmbeddingBagCollection, Embed
 from torchrec_amd.modules.mc_modules import ManagedCollisionCollection
 from torchrec_amd.sparse.jagged_tensor import JaggedTensor, KeyedJaggedTensor, KeyedTensor
 
+Embeddings = Union[KeyedTensor, Dict[str, JaggedTensor]]
+
 
 class BaseManagedCollisionEmbeddingCollection(nn.Module):
-    def __init__(
-        self,
-        embedding_module: Union[EmbeddingBagCollection, EmbeddingCollection],
-        managed_collision_collection: ManagedCollisionCollection,
-        return_remapped_features: bool = False,
-        allow_in_place_embed_weight_update: bool = False,
-    ) -> None:
+    """``forward(kjt) -> (embeddings, remapped kjt or None)``."""
+
+    def __init__(self, embedding_module: Union[EmbeddingBagCollection, EmbeddingCollection],
+                 managed_collision_collection: ManagedCollisionCollection, return_remapped_features: bool = False,
+                 allow_in_place_embed_weight_update: bool = False) -> None:
         super().__init__()
+        pooled = isinstance(embedding_module, EmbeddingBagCollection)
+        configs = embedding_module.embedding_bag_configs() if pooled else embedding_module.embedding_configs()
+        if configs != managed_collision_collection.embedding_configs():
+            raise AssertionError(
+                "Embedding Collection and Managed Collision Collection must contain the same Embedding Configs"
+            )
+        self._embedding_module = embedding_module
         self._managed_collision_collection = managed_collision_collection
         self._return_remapped_features = return_remapped_features
+        # eviction (the only user of this flag) is a training-time step and is not built
         self._allow_in_place_embed_weight_update = allow_in_place_embed_weight_update
-        self._embedding_module = embedding_module
-        configs = (
-            embedding_module.embedding_bag_configs()
-            if isinstance(embedding_module, EmbeddingBagCollection)
-            else embedding_module.embedding_configs()
-        )
-        assert (
-            configs == managed_collision_collection.embedding_configs()
-        ), "Embedding Collection and Managed Collision Collection must contain the same Embedding Configs"
 
-    def forward(
-        self, features: KeyedJaggedTensor
-    ) -> Tuple[Union[KeyedTensor, Dict[str, JaggedTensor]], Optional[KeyedJaggedTensor]]:
-        features = self._managed_collision_collection(features)
-        res = self._embedding_module(features)
-        return (res, features) if self._return_remapped_features else (res, None)
+    def forward(self, features: KeyedJaggedTensor) -> Tuple[Embeddings, Optional[KeyedJaggedTensor]]:
+        remapped = self._managed_collision_collection(features)
+        return self._embedding_module(remapped), (remapped if self._return_remapped_features else None)
 
 
 class ManagedCollisionEmbeddingCollection(BaseManagedCollisionEmbeddingCollection):
-    def __init__(
-        self,
-        embedding_collection: EmbeddingCollection,
-        managed_collision_collection: ManagedCollisionCollection,
-        return_remapped_features: bool = False,
-        allow_in_place_embed_weight_update: bool = False,
-    ) -> None:
-        super().__init__(
-            embedding_collection, managed_collision_collection, return_remapped_features,
-            allow_in_place_embed_weight_update,
-        )
+    """Sequence embeddings (EmbeddingCollection) behind the remap."""
+
+    def __init__(self, embedding_collection: EmbeddingCollection,
+                 managed_collision_collection: ManagedCollisionCollection, return_remapped_features: bool = False,
+                 allow_in_place_embed_weight_update: bool = False) -> None:
+        super().__init__(embedding_collection, managed_collision_collection, return_remapped_features,
+                         allow_in_place_embed_weight_update)
 
     @property
     def _embedding_collection(self) -> EmbeddingCollection:
@@ -61,17 +53,13 @@ class ManagedCollisionEmbeddingCollection(BaseManagedCollisionEmbeddingCollectio
 
 
 class ManagedCollisionEmbeddingBagCollection(BaseManagedCollisionEmbeddingCollection):
-    def __init__(
-        self,
-        embedding_bag_collection: EmbeddingBagCollection,
-        managed_collision_collection: ManagedCollisionCollection,
-        return_remapped_features: bool = False,
-        allow_in_place_embed_weight_update: bool = False,
-    ) -> None:
-        super().__init__(
-            embedding_bag_collection, managed_collision_collection, return_remapped_features,
-            allow_in_place_embed_weight_update,
-        )
+    """Pooled embeddings (EmbeddingBagCollection) behind the remap."""
+
+    def __init__(self, embedding_bag_collection: EmbeddingBagCollection,
+                 managed_collision_collection: ManagedCollisionCollection, return_remapped_features: bool = False,
+                 allow_in_place_embed_weight_update: bool = False) -> None:
+        super().__init__(embedding_bag_collection, managed_collision_collection, return_remapped_features,
+                         allow_in_place_embed_weight_update)
 
     @property
     def _embedding_bag_collection(self) -> EmbeddingBagCollection:
