@@ -30,10 +30,7 @@ def _get_batching_hinted_output(lengths: torch.Tensor, output: torch.Tensor) -> 
 
 
 def _permute_indices(indices: List[int], permute: List[int]) -> List[int]:
-    permuted = [0] * len(indices)
-    for i, p in enumerate(permute):
-        permuted[i] = indices[p]
-    return permuted
+    return [indices[p] for p in permute]
 
 
 def construct_jagged_tensors_inference(
@@ -48,34 +45,31 @@ def construct_jagged_tensors_inference(
 ) -> Dict[str, JaggedTensor]:
     """``embeddings`` [L, D], ``lengths`` [F, B] -> {name: JaggedTensor}.
 
-    Each JaggedTensor's values are a row range (view) of ``embeddings``.  The
-    per-feature row counts are reduced on the device and fetched with a single
-    F-element copy.
+    Each JaggedTensor's values are a row range (view) of ``embeddings``; a name
+    that occurs several times (column-wise shards of one feature) gets its row
+    ranges concatenated along dim 1, in the order ``features_to_permute_indices``
+    gives.  The per-feature row counts are reduced on the device and fetched
+    with a single F-element copy.
     """
     with torch.profiler.record_function("## construct_jagged_tensors_inference ##"):
         if reverse_indices is not None:
             embeddings = torch.index_select(embeddings, 0, reverse_indices.to(torch.int32))
         elif remove_padding:
             embeddings = _slice_1d_tensor(embeddings, 0, int(lengths.sum().item()))
-        F, B = lengths.shape
-        length_per_key: List[int] = ops.length_per_key(lengths.reshape(-1), F, B)
-        lengths_tuple = torch.unbind(lengths, dim=0)
-        embeddings_list = torch.split(embeddings, length_per_key, dim=0)
-        values_list = torch.split(values, length_per_key) if need_indices else None
-        key_indices = defaultdict(list)
-        for i, key in enumerate(embedding_names):
-            key_indices[key].append(i)
-        ret: Dict[str, JaggedTensor] = {}
-        for key, indices in key_indices.items():
-            if features_to_permute_indices and key in features_to_permute_indices:
-                indices = _permute_indices(indices, features_to_permute_indices[key])
-            ret[key] = JaggedTensor(
-                lengths=lengths_tuple[indices[0]],
-                values=(
-                    embeddings_list[indices[0]]
-                    if len(indices) == 1
-                    else torch.cat([embeddings_list[i] for i in indices], dim=1)
-                ),
-                weights=values_list[indices[0]] if values_list is not None else None,
+        num_features, batch = lengths.shape
+        rows_per_feature: List[int] = ops.length_per_key(lengths.reshape(-1), num_features, batch)
+        row_ranges = torch.split(embeddings, rows_per_feature, dim=0)
+        id_ranges = torch.split(values, rows_per_feature) if need_indices else None
+        positions: Dict[str, List[int]] = defaultdict(list)
+        for pos, name in enumerate(embedding_names):
+            positions[name].append(pos)
+        out: Dict[str, JaggedTensor] = {}
+        for name, where in positions.items():
+            if features_to_permute_indices and name in features_to_permute_indices:
+                where = _permute_indices(where, features_to_permute_indices[name])
+            first = where[0]
+            rows = row_ranges[first] if len(where) == 1 else torch.cat([row_ranges[w] for w in where], dim=1)
+            out[name] = JaggedTensor(
+                values=rows, lengths=lengths[first], weights=None if id_ranges is None else id_ranges[first]
             )
-        return ret
+        return out
