@@ -698,6 +698,11 @@ class EmbeddingCollection(EmbeddingCollectionInterface, ModuleNoCopyMixin, _Feat
         offsets = features.offsets()
         lengths = features.lengths().view(len(kjt_keys), -1) if kjt_keys else features.lengths()
         L = indices.numel()
+        # Row ranges of the input keys: one small device-to-host copy.  Asked for
+        # before the lookup is launched, so that the host waits here only for
+        # work that is already queued and then builds the output views while
+        # the lookup runs.
+        offset_per_key = features.offset_per_key()
         lookup = torch.empty((L, self._embedding_dim), dtype=self._output_dtype, device=indices.device)
         f0 = 0
         for emb_module, n_feat in zip(self._emb_modules, self._feature_splits):
@@ -711,8 +716,6 @@ class EmbeddingCollection(EmbeddingCollectionInterface, ModuleNoCopyMixin, _Feat
             f0 += n_feat
         if getattr(self, MODULE_ATTR_USE_BATCHING_HINTED_OUTPUT, True):
             lookup = _get_batching_hinted_output(lengths=lengths, output=lookup)
-        # Row ranges of the input keys (one small device-to-host copy).
-        offset_per_key = features.offset_per_key()
         lengths_rows = torch.unbind(lengths, dim=0) if kjt_keys else ()
         feature_embeddings: Dict[str, JaggedTensor] = {}
         f = 0
