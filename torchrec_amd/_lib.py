@@ -120,18 +120,17 @@ def require_gpu(t: torch.Tensor, what: str) -> None:
         )
 
 
-def ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
-    if t is None:
-        return ctypes.c_void_p(0)
-    return ctypes.c_void_p(t.data_ptr())
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    """Device address of ``t`` as ctypes takes it for a ``void*`` argument (None = NULL)."""
+    return None if t is None else t.data_ptr()
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
-def current_stream(device: torch.device) -> ctypes.c_void_p:
-    """The hipStream_t torch currently launches on for ``device``."""
+def current_stream(device: torch.device) -> int:
+    """The hipStream_t torch currently launches on for ``device`` (as an integer; 0 = null stream)."""
     if _raw_stream is not None:  # no Stream object is built on this route
         idx = device.index if device.index is not None else torch.cuda.current_device()
-        return ctypes.c_void_p(_raw_stream(idx))
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+        return _raw_stream(idx)
+    return torch.cuda.current_stream(device).cuda_stream

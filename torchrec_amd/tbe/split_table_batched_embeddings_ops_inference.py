@@ -132,6 +132,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self.weights_size: int = total
         self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
         self._identity_positions: Tuple[int, ...] = tuple(range(len(self.feature_table_map)))
+        self._num_keys: Dict[Tuple[int, ...], int] = {}
         self._workspace: Optional[Tensor] = None  # scratch of forward(offsets=None, lengths=...)
         self._weights_initialized = False
         self.weight_initialized = False
@@ -147,6 +148,13 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             self._weights_initialized = True
             self.weight_initialized = True
             self._drop_plan()
+
+    def _num_keys_of(self, positions: Tuple[int, ...]) -> int:
+        """Smallest number of KJT keys that covers ``positions`` (remembered per placement)."""
+        n = self._num_keys.get(positions)
+        if n is None:
+            n = self._num_keys[positions] = max(positions) + 1
+        return n
 
     def _rows_view(self, t: int) -> Tensor:
         off, r, rb = self.weights_physical_offsets[t], self.rows[t], self.row_bytes[t]
@@ -309,7 +317,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             assert F > 0 and (offsets.numel() - 1) % F == 0, "offsets must have F * B + 1 entries"
             batch_size = (offsets.numel() - 1) // F
         B = int(batch_size)
-        n_keys = (max(positions) + 1) if positions else F
+        n_keys = F if positions is None else self._num_keys_of(positions)
         if offsets is None:
             assert B == 0 or lengths.numel() % B == 0, "lengths must have K * B entries"
             k_total = lengths.numel() // B if B else n_keys
@@ -336,7 +344,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             else:
                 assert out.shape[0] >= B and out.shape[1] >= out_col + self.total_D
         out_stride = out.stride(0)
-        out_ptr = ctypes.c_void_p(out.data_ptr() + out_col * out.element_size())
+        out_ptr = out.data_ptr() + out_col * out.element_size()
         i64 = int(indices.dtype == torch.int64)
         if offsets is None:
             ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
