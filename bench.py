@@ -387,6 +387,10 @@ def main():
     outs = [forward(i) for i in range(NB)]
     torch.cuda.synchronize()
     graphs = None
+    if args.mode == "graph" and not wl["pooled"]:
+        print("bench.py: --mode graph needs a forward without host reads; the sequence collection fetches its "
+              "per-feature row counts on the host (as the reference does), use --mode eager", file=sys.stderr)
+        sys.exit(2)
     if args.mode == "graph":
         graphs, gouts = [], []
         s = torch.cuda.Stream()
