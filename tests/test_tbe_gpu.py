@@ -164,7 +164,7 @@ def test_feature_positions_and_out_columns():
 
 
 def test_config1_shape_full():
-    """BASELINE config 1 at full size: 8 tables x 100k x 64 int8, B=512, L=20, SUM, fp16 out."""
+    """The smallest benchmark workload at full size: 8 tables x 100k x 64 int8, B=512, L=20, SUM, fp16 out."""
     rng = np.random.default_rng(1001)
     T, rows, dim, B = 8, 100_000, 64, 512
     specs = [(O.INT8, rows, dim)] * T
