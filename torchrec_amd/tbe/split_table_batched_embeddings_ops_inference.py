@@ -133,7 +133,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
         self._identity_positions: Tuple[int, ...] = tuple(range(len(self.feature_table_map)))
         self._num_keys: Dict[Tuple[int, ...], int] = {}
-        self._workspace: Optional[Tensor] = None  # scratch of forward(offsets=None, lengths=...)
+        self._workspace: Dict[int, Tensor] = {}  # per stream: scratch of forward(offsets=None, lengths=...)
         self._weights_initialized = False
         self.weight_initialized = False
         self.register_buffer("weights_dev", torch.empty(0, dtype=torch.uint8, device=device), persistent=False)
@@ -348,13 +348,16 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         i64 = int(indices.dtype == torch.int64)
         if offsets is None:
             ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
-            if self._workspace is None or self._workspace.numel() < ws_bytes or self._workspace.device != dev:
-                self._workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+            stream = _lib.current_stream(dev)
+            # one scratch buffer per stream: calls queued on different streams must not share it
+            ws = self._workspace.get(stream)
+            if ws is None or ws.numel() < ws_bytes or ws.device != dev:
+                ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
             _lib.check(
                 _lib.lib().tra_tbe_forward_lengths(
                     self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices), _lib.ptr(lengths),
                     i64, _lib.ptr(psw), B, k_total, L, int(self.pooling_mode),
-                    self.output_dtype, out_ptr, out_stride, _lib.ptr(self._workspace), _lib.current_stream(dev),
+                    self.output_dtype, out_ptr, out_stride, ws.data_ptr(), stream,
                 )
             )
         else:
