@@ -31,6 +31,13 @@
  *   oracle_bucketize          pure-Python block_bucketize_ref restated in the
  *                             test (distributed/tests/test_utils.py:299-466).
  *
+ * Parity unpinned (nothing in the reference, fbgemm or the mathematics fixes
+ * them; the oracle's choice is stated, not checked):
+ *   - a -1 id in the sequence (no-bag) lookup writes a row of zeros; fbgemm's
+ *     CPU no-bag kernels reject such an input instead.
+ *   - an id outside [0, rows) other than -1 is skipped and reported through
+ *     the return value; fbgemm_gpu's bounds-check modes are not restated.
+ *
  * Build: gcc -O2 -ffp-contract=off -shared -fPIC (see oracle/Makefile).
  * -ffp-contract=off matters: the "acc + bias" add must not fuse with anything.
  */
