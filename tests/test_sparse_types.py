@@ -162,3 +162,64 @@ def test_from_jt_dict_and_concat(device):
     cat = KeyedJaggedTensor.concat([a, b])
     assert cat.keys() == kjt.keys() and torch.equal(cat.values(), kjt.values())
     assert cat.length_per_key() == [3, 5]
+
+
+def test_kjt_equality_cases():
+    """kjt_is_equal on the cases of the reference's test_equality
+    (torchrec/sparse/tests/test_keyed_jagged_tensor.py:892-968)."""
+    from torchrec_amd.sparse.jagged_tensor import kjt_is_equal
+
+    values = torch.Tensor([1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0])
+    weights = torch.Tensor([1.0, 0.5, 1.5, 1.0, 0.5, 1.0, 1.0, 1.5])
+    keys = ["index_0", "index_1"]
+    offsets = torch.IntTensor([0, 0, 2, 2, 3, 4, 5, 5, 8])
+    lengths = torch.IntTensor([0, 2, 0, 1, 1, 1, 0, 3])
+    kt = KeyedJaggedTensor.from_offsets_sync(values=values, keys=keys, offsets=offsets)
+    assert kjt_is_equal(kt, KeyedJaggedTensor.from_lengths_sync(values=values, keys=keys, lengths=lengths))
+    assert not kjt_is_equal(kt, KeyedJaggedTensor(values=values, keys=["index_1", "index_0"], offsets=offsets))
+    other = torch.Tensor([10.0, 4.0, 2.0, 5.0, 2.0, 6.0, 9.0, 8.0])
+    assert not kjt_is_equal(kt, KeyedJaggedTensor(values=other, keys=keys, lengths=lengths))
+    assert not kjt_is_equal(kt, KeyedJaggedTensor(values=values, keys=["index_0"], offsets=offsets))
+    assert not kjt_is_equal(kt, KeyedJaggedTensor.from_offsets_sync(values=values, keys=keys, offsets=offsets, weights=weights))
+    a = KeyedJaggedTensor.from_lengths_sync(values=values, keys=keys, lengths=torch.IntTensor([1, 2, 3, 4, 5, 6, 7, 8]))
+    b = KeyedJaggedTensor.from_lengths_sync(values=values, keys=keys, lengths=torch.IntTensor([8, 7, 6, 5, 4, 3, 2, 1]))
+    assert not kjt_is_equal(a, b)
+    c = KeyedJaggedTensor.from_offsets_sync(values=values, keys=keys, offsets=torch.IntTensor([8, 4, 1, 5, 0, 1, 2, 1, 2]))
+    assert not kjt_is_equal(kt, c)
+    assert not kjt_is_equal(kt, "not a kjt")
+
+
+def test_kjt_strings():
+    """str() of a KJT, as the reference prints it (test_keyed_jagged_tensor.py:786-852)."""
+    assert str(KeyedJaggedTensor([], torch.Tensor())) == "KeyedJaggedTensor()\n"
+    one = KeyedJaggedTensor(values=torch.Tensor([1.0]), keys=["key"], offsets=torch.IntTensor([0, 1]))
+    assert str(one) == 'KeyedJaggedTensor({\n    "key": [[1.0]]\n})\n'
+    values = torch.Tensor([1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0])
+    weights = torch.Tensor([1.0, 0.5, 1.5, 1.0, 0.5, 1.0, 1.0, 1.5])
+    keys = ["index_0", "index_1"]
+    offsets = torch.IntTensor([0, 2, 2, 3, 4, 5, 8])
+    assert str(KeyedJaggedTensor(values=values, keys=keys, offsets=offsets)) == (
+        'KeyedJaggedTensor({\n    "index_0": [[1.0, 2.0], [], [3.0]],\n'
+        '    "index_1": [[4.0], [5.0], [6.0, 7.0, 8.0]]\n})\n')
+    assert str(KeyedJaggedTensor(values=values, keys=keys, offsets=offsets, weights=weights)) == (
+        'KeyedJaggedTensor({\n    "index_0": {\n'
+        '        "values": [[1.0, 2.0], [], [3.0]],\n'
+        '        "weights": [[1.0, 0.5], [], [1.5]]\n'
+        '    },\n    "index_1": {\n'
+        '        "values": [[4.0], [5.0], [6.0, 7.0, 8.0]],\n'
+        '        "weights": [[1.0], [0.5], [1.0, 1.0, 1.5]]\n    }\n})\n')
+
+
+def test_kjt_to_dict_and_empty():
+    """to_dict / empty / empty_like (test_keyed_jagged_tensor.py:102-140, 225-290)."""
+    values = torch.Tensor([1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0])
+    weights = torch.Tensor([1.0, 0.5, 1.5, 1.0, 0.5, 1.0, 1.0, 1.5])
+    keys = ["index_0", "index_1"]
+    offsets = torch.IntTensor([0, 2, 2, 3, 4, 5, 8])
+    d = KeyedJaggedTensor(values=values, weights=weights, keys=keys, offsets=offsets).to_dict()
+    assert d["index_0"].offsets().tolist() == [0, 2, 2, 3] and d["index_0"].values().tolist() == [1.0, 2.0, 3.0]
+    assert d["index_1"].offsets().tolist() == [0, 1, 2, 5] and d["index_1"].weights().tolist() == [1.0, 0.5, 1.0, 1.0, 1.5]
+    e = KeyedJaggedTensor.empty()
+    assert e.keys() == [] and e.values().numel() == 0 and e.to_dict() == {}
+    like = KeyedJaggedTensor.empty_like(KeyedJaggedTensor(values=values, weights=weights, keys=keys, offsets=offsets))
+    assert like.keys() == [] and like.values().dtype == values.dtype and like.weights().numel() == 0

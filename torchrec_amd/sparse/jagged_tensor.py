@@ -622,16 +622,25 @@ class KeyedJaggedTensor:
                 t.record_stream(stream)
 
     def __str__(self) -> str:
+        # Same text as the reference prints (jagged_tensor.py:1295-1317, 3081-3108).
         if len(self._keys) == 0:
             return "KeyedJaggedTensor()\n"
         offs = self.offsets().tolist()
         B = self.stride()
+
+        def rows_of(t: torch.Tensor, f: int) -> str:
+            cells = (_values_string(t, offs[f * B + b], offs[f * B + b + 1]) for b in range(B))
+            return "[" + ", ".join(cells) + "]"
+
         parts = []
         for f, key in enumerate(self._keys):
-            rows = ", ".join(
-                _values_string(self._values, offs[f * B + b], offs[f * B + b + 1]) for b in range(B)
-            )
-            parts.append(f'    "{key}": [{rows}]')
+            if self._weights is None:
+                parts.append(f'    "{key}": {rows_of(self._values, f)}')
+            else:
+                parts.append(
+                    f'    "{key}": {{\n        "values": {rows_of(self._values, f)},\n'
+                    f'        "weights": {rows_of(self._weights, f)}\n    }}'
+                )
         return "KeyedJaggedTensor({\n" + ",\n".join(parts) + "\n})\n"
 
 
