@@ -1,0 +1,329 @@
+"""Per-shard lookup modules (QuantBatchedEmbeddingBag / QuantBatchedEmbedding,
+torchrec/distributed/quant_embedding_kernel.py:248-663).
+
+Host part: config helpers, fused-parameter readers, operator specs and the
+state-dict view.  GPU part: one module against the oracle, the lengths form
+against the offsets form, and the two ways a table is cut for sharded
+inference replayed on one GPU -- column shards whose outputs concatenate to the
+unsharded output bit for bit, and row shards fed by the bucketized KJT whose
+partial sums add up to it (sequence rows come back in input order through the
+unbucketize permute, bit for bit)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+from torch.distributed._shard.metadata import ShardMetadata
+from torch.distributed._shard.sharded_tensor.metadata import ShardedTensorMetadata
+
+from torchrec_amd import KeyedJaggedTensor
+from torchrec_amd.distributed import fused_params as FP
+from torchrec_amd.distributed.embedding_types import (
+    EmbeddingComputeKernel,
+    GroupedEmbeddingConfig,
+    ShardedEmbeddingTable,
+    compute_kernel_to_embedding_location,
+)
+from torchrec_amd.distributed.quant_embedding_kernel import (
+    IntNBitTableBatchedEmbeddingBagsCodegenWithLength,
+    QuantBatchedEmbedding,
+    QuantBatchedEmbeddingBag,
+    _copy_config,
+    _get_runtime_device,
+)
+from torchrec_amd.modules.embedding_configs import DataType, PoolingType
+from torchrec_amd.tbe.enums import BoundsCheckMode, EmbeddingLocation, PoolingMode, SparseType
+
+
+def table(name, rows, dim, feats, data_type=DataType.INT4, local_rows=None, local_cols=None, offsets=None,
+          pooling=PoolingType.SUM, weighted=False):
+    local_rows = rows if local_rows is None else local_rows
+    local_cols = dim if local_cols is None else local_cols
+    return ShardedEmbeddingTable(
+        num_embeddings=rows, embedding_dim=dim, name=name, data_type=data_type, feature_names=list(feats),
+        pooling=pooling, is_weighted=weighted, embedding_names=list(feats),
+        compute_kernel=EmbeddingComputeKernel.QUANT, local_rows=local_rows, local_cols=local_cols,
+        local_metadata=ShardMetadata(shard_offsets=list(offsets or [0, 0]), shard_sizes=[local_rows, local_cols],
+                                     placement="rank:0/cuda:0"),
+    )
+
+
+def group(tables, pooling=PoolingType.SUM, weighted=False, data_type=DataType.INT4, fused_params=None):
+    return GroupedEmbeddingConfig(data_type=data_type, pooling=pooling, is_weighted=weighted,
+                                  has_feature_processor=False, compute_kernel=EmbeddingComputeKernel.QUANT,
+                                  embedding_tables=tables, fused_params=fused_params)
+
+
+SPLIT = {FP.FUSED_PARAM_QUANT_STATE_DICT_SPLIT_SCALE_BIAS: True}
+
+
+# ---- host ----------------------------------------------------------------------
+
+def test_grouped_config_helpers():
+    g = group([table("t0", 100, 32, ["a", "b"], local_cols=16), table("t1", 50, 64, ["c"])])
+    assert g.num_features() == 3
+    assert g.feature_names() == ["a", "b", "c"] and g.embedding_names() == ["a", "b", "c"]
+    assert g.table_names() == ["t0", "t1"]
+    assert g.feature_hash_sizes() == [100, 100, 50]
+    assert g.embedding_dims() == [16, 16, 64] and g.dim_sum() == 96
+    assert [m.shard_sizes for m in g.embedding_shard_metadata()] == [[100, 16], [100, 16], [50, 64]]
+    assert not g.is_using_virtual_table()
+
+
+def test_compute_kernel_locations():
+    loc = compute_kernel_to_embedding_location
+    assert loc(EmbeddingComputeKernel.QUANT) == EmbeddingLocation.DEVICE
+    assert loc(EmbeddingComputeKernel.QUANT_UVM) == EmbeddingLocation.MANAGED
+    assert loc(EmbeddingComputeKernel.QUANT_UVM_CACHING) == EmbeddingLocation.MANAGED_CACHING
+    with pytest.raises(ValueError):
+        loc(EmbeddingComputeKernel.CUSTOMIZED_KERNEL)
+
+
+def test_fused_param_readers():
+    assert not FP.is_fused_param_register_tbe(None) and not FP.is_fused_param_register_tbe({})
+    fused = {
+        FP.FUSED_PARAM_REGISTER_TBE_BOOL: True,
+        FP.FUSED_PARAM_QUANT_STATE_DICT_SPLIT_SCALE_BIAS: True,
+        FP.FUSED_PARAM_TBE_ROW_ALIGNMENT: 8,
+        FP.FUSED_PARAM_BOUNDS_CHECK_MODE: BoundsCheckMode.NONE,
+        FP.FUSED_PARAM_LENGTHS_TO_OFFSETS_LOOKUP: True,
+        FP.FUSED_PARAM_SSD_TABLE_LIST: ["x"],
+        "output_dtype": SparseType.FP32,
+    }
+    assert FP.is_fused_param_register_tbe(fused)
+    assert FP.is_fused_param_quant_state_dict_split_scale_bias(fused)
+    assert FP.get_fused_param_tbe_row_alignment(fused) == 8 and FP.get_fused_param_tbe_row_alignment(None) is None
+    assert FP.fused_param_bounds_check_mode(fused) == BoundsCheckMode.NONE
+    assert FP.fused_param_lengths_to_offsets_lookup(fused) and not FP.fused_param_lengths_to_offsets_lookup({})
+    assert FP.tbe_fused_params(fused) == {"output_dtype": SparseType.FP32}
+    assert FP.tbe_fused_params(None) is None and FP.tbe_fused_params({}) is None
+
+
+def test_copy_config_packs_widths():
+    t = table("t0", 100, 128, ["a"], data_type=DataType.FP32)
+    t.global_metadata = ShardedTensorMetadata(
+        shards_metadata=[t.local_metadata, ShardMetadata(shard_offsets=[0, 128], shard_sizes=[100, 128],
+                                                         placement="rank:1/cuda:1")],
+        size=torch.Size([100, 256]))
+    g = group([t], data_type=DataType.FP32)
+    q = _copy_config(g, DataType.INT4, SparseType.INT4, torch.device("cuda"))
+    qt = q.embedding_tables[0]
+    assert q.data_type == DataType.INT4
+    assert qt.local_cols == 80  # 4-byte header + 64 payload bytes, rounded up to 16
+    assert qt.local_metadata.shard_sizes == [100, 80]
+    assert [s.shard_sizes for s in qt.global_metadata.shards_metadata] == [[100, 80], [100, 80]]
+    assert tuple(qt.global_metadata.size) == (100, 160)
+    assert g.embedding_tables[0].local_cols == 128  # the original is left alone
+    host = _copy_config(g, DataType.INT8, SparseType.INT8, torch.device("cpu"))
+    assert host.embedding_tables[0].local_cols == 132  # packed: no alignment on the host
+
+
+def test_runtime_device_from_placements():
+    g = group([table("t0", 10, 16, ["a"])])
+    assert _get_runtime_device(torch.device("cpu"), g) == torch.device("cpu")
+    assert _get_runtime_device(None, g) == torch.device("cuda")
+    assert _get_runtime_device(torch.device("meta"), g) == torch.device("cuda")
+    h = copy.deepcopy(g)
+    h.embedding_tables[0].local_metadata.placement = torch.distributed._remote_device("rank:0/cpu")
+    assert _get_runtime_device(None, h) == torch.device("cpu")
+
+
+@pytest.mark.parametrize("cls", [QuantBatchedEmbeddingBag, QuantBatchedEmbedding])
+def test_operator_specs_and_state_dict_view(cls):
+    tables = [table("t0", 40, 128, ["a", "b"], local_rows=20, local_cols=64, offsets=[20, 64]),
+              table("t1", 10, 32, ["c"], data_type=DataType.INT8)]
+    # whole rows in the state dict: the operator gets the table's own width
+    m = cls(group(tables), device=torch.device("cpu"))
+    op = m.emb_module
+    assert [(s[0], s[1], s[2], s[3]) for s in op.embedding_specs] == [
+        ("t0", 20, 128, SparseType.INT4), ("t1", 10, 32, SparseType.INT8)]
+    assert all(s[4] == EmbeddingLocation.HOST for s in op.embedding_specs)
+    assert op.feature_table_map == [0, 0, 1] and op.feature_names_per_table == [["a", "b"], ["c"]]
+    assert op.row_alignment == 1
+    assert op.pooling_mode == (PoolingMode.SUM if cls is QuantBatchedEmbeddingBag else PoolingMode.NONE)
+    named = dict(m.named_buffers(prefix="x"))
+    assert list(named) == ["x.t0.weight", "x.t1.weight"]
+    assert named["x.t0.weight"].shape == (20, 68) and named["x.t1.weight"].shape == (10, 36)
+    assert m.get_tbes_to_register() == {op: m.config}
+    assert FP.get_tbes_to_register_from_iterable([m, torch.nn.Linear(1, 1)]) == {op: m.config}
+    # scale and bias apart: the shard's width, three buffers per table, views of the store
+    m = cls(group(tables), device=torch.device("cpu"), fused_params=SPLIT)
+    op = m.emb_module
+    assert [s[2] for s in op.embedding_specs] == [64, 32]
+    named = dict(m.named_buffers())
+    assert list(named) == ["t0.weight", "t0.weight_qscale", "t0.weight_qbias",
+                           "t1.weight", "t1.weight_qscale", "t1.weight_qbias"]
+    assert named["t0.weight"].shape == (20, 32) and named["t0.weight"].dtype == torch.uint8
+    assert named["t0.weight_qscale"].shape == (20, 1) and named["t0.weight_qscale"].dtype == torch.float16
+    named["t1.weight_qbias"].fill_(2.0)
+    assert float(m.split_embedding_weights()[1][2][3, 0]) == 2.0
+    assert named["t1.weight"].untyped_storage().data_ptr() == op.weights_dev.untyped_storage().data_ptr()
+
+
+def test_lengths_flag_and_bounds_check_mode():
+    g = group([table("t0", 10, 16, ["a"])])
+    m = QuantBatchedEmbeddingBag(g, device=torch.device("cpu"))
+    assert not m.lengths_to_tbe and type(m.emb_module).__name__ == "IntNBitTableBatchedEmbeddingBagsCodegen"
+    assert m.emb_module.bounds_check_mode_int == int(BoundsCheckMode.WARNING)
+    m = QuantBatchedEmbeddingBag(g, device=torch.device("cpu"), fused_params={
+        FP.FUSED_PARAM_LENGTHS_TO_OFFSETS_LOOKUP: True, FP.FUSED_PARAM_BOUNDS_CHECK_MODE: BoundsCheckMode.NONE})
+    assert m.lengths_to_tbe and isinstance(m.emb_module, IntNBitTableBatchedEmbeddingBagsCodegenWithLength)
+    assert m.emb_module.bounds_check_mode_int == int(BoundsCheckMode.NONE)
+    virtual = copy.deepcopy(g)
+    virtual.embedding_tables[0].use_virtual_table = True
+    with pytest.raises(NotImplementedError):
+        QuantBatchedEmbeddingBag(virtual, device=torch.device("cpu"))
+
+
+def test_forward_needs_the_gpu():
+    m = QuantBatchedEmbeddingBag(group([table("t0", 10, 16, ["a"])]), device=torch.device("cpu"))
+    kjt = KeyedJaggedTensor(keys=["a"], values=torch.tensor([1, 2]), lengths=torch.tensor([2]))
+    with pytest.raises(RuntimeError):
+        m(kjt)
+
+
+# ---- GPU -----------------------------------------------------------------------
+
+def _gpu_helpers():
+    import oracle as O
+    from helpers import bits_equal
+    from test_quant_modules_gpu import oracle_store_of, random_kjt
+    return O, bits_equal, oracle_store_of, random_kjt
+
+
+def _fill_random(module, rng):
+    """Random packed bytes with sane fp16 headers (scale in [0.01, 0.02], bias in [-0.1, 0))."""
+    for weight, scale, bias in module.emb_module.split_embedding_weights_with_scale_bias(2):
+        weight.copy_(torch.from_numpy(rng.integers(0, 256, tuple(weight.shape), dtype=np.uint8)))
+        if scale is not None:
+            scale.copy_(torch.from_numpy((0.01 + 0.01 * rng.random(tuple(scale.shape))).astype(np.float16)))
+            bias.copy_(torch.from_numpy((-0.1 * rng.random(tuple(bias.shape))).astype(np.float16)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pooling,weighted", [(PoolingType.SUM, False), (PoolingType.SUM, True), (PoolingType.MEAN, False)])
+def test_pooled_module_matches_oracle_and_lengths_form(pooling, weighted):
+    O, bits_equal, oracle_store_of, random_kjt = _gpu_helpers()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(5)
+    tables = [table("t0", 300, 128, ["a", "b"], pooling=pooling, weighted=weighted),
+              table("t1", 77, 64, ["c"], data_type=DataType.INT8, pooling=pooling, weighted=weighted)]
+    fused = {**SPLIT, "output_dtype": SparseType.FP32}
+    by_offsets = QuantBatchedEmbeddingBag(group(tables, pooling, weighted), device=dev, fused_params=fused)
+    by_lengths = QuantBatchedEmbeddingBag(group(tables, pooling, weighted), device=dev,
+                                          fused_params={**fused, FP.FUSED_PARAM_LENGTHS_TO_OFFSETS_LOOKUP: True,
+                                                        FP.FUSED_PARAM_REGISTER_TBE_BOOL: True})
+    _fill_random(by_offsets, rng)
+    by_lengths.emb_module.weights_dev.copy_(by_offsets.emb_module.weights_dev)
+    kjt = random_kjt(rng, ["a", "b", "c"], [300, 300, 77], B=37, max_len=9, weighted=weighted)
+    got = by_offsets(kjt)
+    assert got.shape == (37, 128 + 128 + 64) and got.dtype == torch.float32
+    op = by_offsets.emb_module
+    want = O.tbe_forward(oracle_store_of(op), op.feature_table_map, 37, kjt.values().cpu().numpy(),
+                         kjt.offsets().cpu().numpy().astype(np.int64),
+                         kjt.weights().cpu().numpy() if weighted else None, int(op.pooling_mode), O.FP32)
+    assert bits_equal(got.cpu().numpy(), want) == 0
+    assert torch.equal(by_lengths(kjt), got)
+
+
+@pytest.mark.gpu
+def test_column_shards_concatenate_to_the_whole_table():
+    O, bits_equal, oracle_store_of, random_kjt = _gpu_helpers()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(6)
+    rows, dim, shards = 500, 256, 4
+    width = dim // shards
+    whole = QuantBatchedEmbeddingBag(group([table("t", rows, dim, ["f"], data_type=DataType.INT8)]),
+                                     device=dev, fused_params=SPLIT)
+    _fill_random(whole, rng)
+    payload, scale, bias = whole.emb_module.split_embedding_weights_with_scale_bias(2)[0]
+    kjt = random_kjt(rng, ["f"], [rows], B=64, max_len=20)
+    parts = []
+    for s in range(shards):
+        shard = QuantBatchedEmbeddingBag(
+            group([table("t", rows, dim, ["f"], data_type=DataType.INT8, local_cols=width, offsets=[0, s * width])]),
+            device=dev, fused_params=SPLIT, shard_index=s)
+        assert shard.emb_module.dims == [width]
+        w, sc, bi = shard.emb_module.split_embedding_weights_with_scale_bias(2)[0]
+        w.copy_(payload[:, s * width:(s + 1) * width])  # every column shard keeps the row's scale and bias
+        sc.copy_(scale)
+        bi.copy_(bias)
+        parts.append(shard(kjt))
+    assert torch.equal(torch.cat(parts, dim=1), whole(kjt))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sequence", [False, True])
+def test_row_shards_fed_by_the_bucketized_kjt(sequence):
+    from torchrec_amd.sparse.bucketize import bucketize_kjt_inference
+    O, bits_equal, oracle_store_of, random_kjt = _gpu_helpers()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(7)
+    rows, dim, shards = 1000, 64, 4
+    block = rows // shards
+    cls = QuantBatchedEmbedding if sequence else QuantBatchedEmbeddingBag
+    fused = {**SPLIT, "output_dtype": SparseType.FP32}
+    feats = ["f", "g"]
+    whole = cls(group([table("t", rows, dim, feats)]), device=dev, fused_params=fused)
+    _fill_random(whole, rng)
+    full_rows = whole.emb_module.split_embedding_weights_with_scale_bias(0)[0][0]
+    kjt = random_kjt(rng, feats, [rows, rows], B=48, max_len=12)
+    want = whole(kjt)
+    bucketized, unbucketize, bucket_of_id = bucketize_kjt_inference(
+        kjt, shards, torch.tensor([block, block]), is_sequence=sequence)
+    per_shard = bucketized.split([len(feats)] * shards)
+    outs = []
+    for s in range(shards):
+        shard = cls(group([table("t", rows, dim, feats, local_rows=block, offsets=[s * block, 0])]),
+                    device=dev, fused_params=fused, shard_index=s)
+        shard.emb_module.split_embedding_weights_with_scale_bias(0)[0][0].copy_(full_rows[s * block:(s + 1) * block])
+        assert per_shard[s].keys() == feats
+        outs.append(shard(per_shard[s]))
+    if sequence:
+        # rows of all shards, shard-major, back into the order of the input ids
+        assert torch.equal(torch.cat(outs, dim=0)[unbucketize.long()], want)
+        assert torch.equal(bucket_of_id, torch.div(kjt.values(), block, rounding_mode="floor"))
+    else:
+        # partial sums per shard add up to the whole bag; the order of addition
+        # differs from the single-table loop, hence a tolerance (1e-5 relative)
+        total = torch.stack(outs).sum(dim=0)
+        torch.testing.assert_close(total, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_from_float_module():
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(8)
+
+    class FloatGroup(torch.nn.Module):
+        def __init__(self, config):
+            super().__init__()
+            self._config = config
+            self.tables = torch.nn.ParameterList(
+                [torch.nn.Parameter(0.1 * torch.randn(t.local_rows, t.local_cols, device=dev))
+                 for t in config.embedding_tables])
+
+        @property
+        def config(self):
+            return self._config
+
+    torch.manual_seed(8)
+    g = group([table("t0", 60, 32, ["a"], data_type=DataType.FP32), table("t1", 40, 32, ["b"], data_type=DataType.FP32)],
+              data_type=DataType.FP32)
+    fl = FloatGroup(g)
+    fl.qconfig = torch.quantization.QConfig(activation=torch.quantization.PlaceholderObserver.with_args(dtype=torch.float),
+                                            weight=torch.quantization.PlaceholderObserver.with_args(dtype=torch.qint8))
+    q = QuantBatchedEmbeddingBag.from_float(fl)
+    assert q.config.data_type == DataType.INT8 and q.config.embedding_tables[0].local_cols == 48
+    assert q.emb_module.dims == [32, 32] and [str(t) for t in q.emb_module.weight_tys] == ["int8", "int8"]
+    _, _, _, random_kjt = _gpu_helpers()
+    kjt = random_kjt(rng, ["a", "b"], [60, 40], B=16, max_len=6)
+    got = q(kjt).float()
+    offs = kjt.offsets().cpu().numpy()
+    ids = kjt.values().cpu().numpy()
+    want = torch.zeros(16, 64)
+    for f, w in enumerate(fl.tables):
+        for b in range(16):
+            lo, hi = offs[f * 16 + b], offs[f * 16 + b + 1]
+            want[b, f * 32:(f + 1) * 32] = w.detach().cpu()[ids[lo:hi]].sum(dim=0)
+    torch.testing.assert_close(got.cpu(), want, atol=0.1, rtol=0)

@@ -159,8 +159,13 @@ def block_bucketize_sparse_features(
         raise NotImplementedError("bucketize_pos is not supported")
     _lib.require_gpu(lengths, "block_bucketize_sparse_features")
     _check_int(lengths, "lengths")
-    if indices.dtype != lengths.dtype:
-        raise TypeError("indices and lengths must share an integer dtype")
+    _check_int(indices, "indices")
+    # The kernels take ids and lengths in one width; lengths of another width
+    # (a KJT usually carries int32 lengths beside int64 ids) are widened or
+    # narrowed on the way in and the new lengths given back in the caller's.
+    lengths_dtype = lengths.dtype
+    if indices.dtype != lengths_dtype:
+        lengths = lengths.to(indices.dtype)
     dev = lengths.device
     l = _lib.lib()
     stream = _lib.current_stream(dev)
@@ -197,6 +202,8 @@ def block_bucketize_sparse_features(
             _lib.ptr(new_weights), _lib.ptr(unbucketize), stream,
         )
     )
+    if new_lengths.dtype != lengths_dtype:
+        new_lengths = new_lengths.to(lengths_dtype)
     return new_lengths, new_indices, new_weights, None, unbucketize
 
 

@@ -97,3 +97,13 @@ class EmbeddingLocation(enum.IntEnum):
     MANAGED_CACHING = 2
     HOST = 3
     MTIA = 4
+
+
+class BoundsCheckMode(enum.IntEnum):
+    """What the lookup does about an id outside its table (fbgemm_gpu's codes;
+    the reference re-exports the enum as torchrec.distributed.types.BoundsCheckMode)."""
+
+    FATAL = 0    # raise
+    WARNING = 1  # report and go on
+    IGNORE = 2   # go on silently
+    NONE = 3     # no check

@@ -26,7 +26,7 @@ import torch
 from torch import nn, Tensor
 
 from torchrec_amd import _lib
-from torchrec_amd.tbe.enums import EmbeddingLocation, PoolingMode, SparseType
+from torchrec_amd.tbe.enums import BoundsCheckMode, EmbeddingLocation, PoolingMode, SparseType
 
 _SUPPORTED_WEIGHTS = (SparseType.FP32, SparseType.FP16, SparseType.INT8, SparseType.INT4, SparseType.INT2)
 _TABLE_ALIGNMENT = 256
@@ -63,9 +63,14 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         weight_lists: Optional[List[Tuple[Tensor, Optional[Tensor]]]] = None,
         output_dtype: SparseType = SparseType.FP16,
         row_alignment: Optional[int] = None,
+        uvm_host_mapped: bool = False,
+        feature_names_per_table: Optional[List[List[str]]] = None,
         **unsupported,
     ) -> None:
         super().__init__()
+        # uvm_host_mapped chooses how host-mapped tables are allocated; every
+        # table here lives in HBM, so it has nothing to act on.
+        self.feature_names_per_table = feature_names_per_table
         if index_remapping:
             raise NotImplementedError("index_remapping (pruning hash maps) is not supported")
         for k, v in unsupported.items():
@@ -81,6 +86,9 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self.embedding_specs = embedding_specs
         self.pooling_mode = pooling_mode
         self.output_dtype: int = output_dtype.as_int()
+        # An id outside [0, rows) is skipped (adds nothing) and counted in every
+        # mode; BoundsCheckMode.FATAL also raises after the call, which waits
+        # for the kernel.
         self.bounds_check_mode_int: int = -1 if bounds_check_mode is None else int(bounds_check_mode)
         if output_dtype not in (SparseType.FP32, SparseType.FP16):
             raise NotImplementedError(f"output dtype {output_dtype} (fp32 and fp16 are supported)")
@@ -368,7 +376,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                     self.output_dtype, out_ptr, out_stride, _lib.current_stream(dev),
                 )
             )
-        if os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1":
+        if self.bounds_check_mode_int == int(BoundsCheckMode.FATAL) or os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1":
             bad = self.out_of_range_count()
             if bad:
                 raise IndexError(f"{bad} embedding indices were out of range")
