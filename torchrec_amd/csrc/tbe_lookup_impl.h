@@ -702,6 +702,23 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     front_part = prefix_partial<IdxT>(reinterpret_cast<const IdxT*>(a.offsets),
                                       (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B), blk);
 
+  // Bag q0 + i of the window: where it sits in the offsets (or lengths) array.
+  auto bag_of = [&](int i, int& fi, int& b) -> int64_t {
+    const int q = q0 + i;
+    fi = q / a.B;
+    b = q - fi * a.B;
+    return (int64_t)feat_key_pos(a, sc, fi) * a.B + b;
+  };
+  // The first bag of every thread is requested before anything else: the
+  // barrier below waits for outstanding loads, and this way the bag bounds
+  // and the descriptors share one memory latency instead of queueing up.
+  IdxT first_lo = 0, first_hi = 0;
+  if ((int)threadIdx.x < nb) {
+    int fi, b;
+    const int64_t bag = bag_of(threadIdx.x, fi, b);
+    first_lo = reinterpret_cast<const IdxT*>(a.offsets)[bag];
+    if (!FROM_LENGTHS) first_hi = reinterpret_cast<const IdxT*>(a.offsets)[bag + 1];
+  }
   // Descriptors of the features this window touches, kept in LDS so that a
   // round does not start with two dependent global loads.
   {
@@ -711,18 +728,17 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < nb; i += kCuThreads) {
-    const int q = q0 + i;
-    const int fi = q / a.B;
-    const int b = q - fi * a.B;
-    const int fpos = feat_key_pos(a, sc, fi);
-    const int64_t bag = (int64_t)fpos * a.B + b;
+    int fi, b;
+    const int64_t bag = bag_of(i, fi, b);
+    const bool first = i == (int)threadIdx.x;
     int len;
     if (FROM_LENGTHS) {
-      len = max(0, (int)load_index<IdxT>(a.offsets, bag));
+      len = max(0, (int)(first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag)));
     } else {
-      const int64_t st = load_index<IdxT>(a.offsets, bag);
+      const int64_t st = first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag);
+      const int64_t en = first ? (int64_t)first_hi : load_index<IdxT>(a.offsets, bag + 1);
       s_start[i] = st;
-      len = max(0, (int)(load_index<IdxT>(a.offsets, bag + 1) - st));
+      len = max(0, (int)(en - st));
     }
     s_len[i] = len;
     s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
@@ -839,8 +855,9 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   // Rounds are ordered longest first and dealt to the waves four at a time,
   // alternating direction over the four SIMDs.  (Dealing them in a strict
   // snake over all 16 waves, or evening out the rounds per wave, measured
-  // slower: the waves that finish early leave the CU's memory pipeline to the
-  // ones still running.)
+  // slower, and handing rounds out from a counter as waves become free
+  // measured the same: the waves that finish early leave the CU's memory
+  // pipeline to the ones still running.)
   for (int pass = 0; pass * kCuWaves < rounds; ++pass) {
     const int slot = pass * 4 + (wave >> 2);
     const int r = slot * 4 + ((slot & 1) ? 3 - (wave & 3) : (wave & 3));
