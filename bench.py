@@ -45,6 +45,9 @@ def parse_args():
     p.add_argument("--batches", type=int, default=8, help="distinct id batches rotated through")
     p.add_argument("--mode", default="eager", choices=["graph", "eager"])
     p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
+    p.add_argument("--alt-row-alignment", type=int, default=None,
+                   help="also measure the same workload with this row alignment (default: 64 for c2, i.e. one "
+                        "128-byte line per row; 0 = skip)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline sample")
     p.add_argument("--rocprof-summary", metavar="DIR", default=None,
@@ -348,6 +351,77 @@ def rocprof_summary(root):
             print(f"{len(v):10d} {sum(v) / len(v):20.1f}  {c}  {k}")
 
 
+def measure_alt_layout(args, dev, row_alignment, ref_out):
+    """The same workload (same seeds: same tables, same ids) stored with another
+    row alignment: step time of the module forward, kernel time of its lookup
+    launch, and whether the outputs equal those of the default layout."""
+    import argparse as _ap
+    import torch
+    from torchrec_amd import _lib, KeyedJaggedTensor
+
+    alt = _ap.Namespace(**vars(args))
+    alt.row_alignment = row_alignment
+    wl = build_workload(alt, dev)
+    module, batches, keys = wl["module"], wl["batches"], wl["keys"]
+    NB = len(batches)
+
+    def forward(i):
+        v, l, w = batches[i]
+        return module(KeyedJaggedTensor(keys=keys, values=v, lengths=l, weights=w))
+
+    out0 = forward(0)
+    torch.cuda.synchronize()
+    same = bool(torch.equal(out0.values(), ref_out))
+    steps, warm = args.steps, min(args.warmup, 200)
+    for k in range(warm):
+        forward(k % NB)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        forward(k % NB)
+    torch.cuda.synchronize()
+    el = time.perf_counter() - t0
+    tbe = module._emb_modules[0]
+    lib = _lib.lib()
+    plan = tbe._get_plan(None)
+    stream = _lib.current_stream(dev)
+    kout = out0.values().clone()
+    ws = torch.empty(max(256, lib.tra_tbe_forward_lengths_workspace_bytes(wl["T"], wl["B"], 0)), dtype=torch.uint8, device=dev)
+    info = ctypes.create_string_buffer(4096)
+    _lib.check(lib.tra_tbe_launch_info(plan, wl["B"], batches[0][0].numel(), int(tbe.pooling_mode), wl["T"], info, len(info)))
+    launches = info.value.decode().split("; ")
+
+    def launch(i):
+        v, l, w = batches[i]
+        _lib.check(lib.tra_tbe_forward_lengths(plan, _lib.ptr(tbe.weights_dev), _lib.ptr(v), _lib.ptr(l), 0, _lib.ptr(w),
+                                               wl["B"], wl["T"], v.numel(), int(tbe.pooling_mode), tbe.output_dtype,
+                                               _lib.ptr(kout), kout.stride(0), _lib.ptr(ws), stream))
+
+    for k in range(warm):
+        launch(k % NB)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for k in range(steps):
+        launch(k % NB)
+    e1.record()
+    torch.cuda.synchronize()
+    call_ms = e0.elapsed_time(e1) / steps
+    alg = sum(wl["alg_bytes"][k % NB] for k in range(steps)) / steps
+    lookups = sum(batches[k % NB][0].numel() for k in range(steps))
+    return {
+        "row_alignment": row_alignment,
+        "store_GB": wl["store_bytes"] / 1e9,
+        "value": lookups / el, "unit": "lookups/s", "ms_per_step": el / steps * 1e3,
+        "lookup_call_ms": call_ms, "launches_per_call": launches,
+        "achieved": alg / (call_ms * 1e-3) / 1e9, "frac": alg / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "outputs_equal_default_layout": same,
+        "note": "same tables and ids, rows padded to the given alignment (QuantEmbeddingBagCollection(row_alignment=...)); "
+                "algorithmic bytes unchanged (unpadded rows); lookup_call_ms covers the whole lookup call "
+                "(tra_tbe_forward_lengths), scan kernels included when it is not fused",
+    }
+
+
 def main():
     args = parse_args()
     if args.rocprof_summary:
@@ -614,6 +688,12 @@ def main():
     if other:
         result["eager_value"] = total_lookups / el_other
         result["eager_ms_per_step"] = el_other / args.steps * 1e3
+    alt_ra = args.alt_row_alignment
+    if alt_ra is None:
+        alt_ra = 64 if args.config == "c2" else 0
+    if alt_ra and alt_ra != args.row_alignment and wl["pooled"]:
+        print(f"[bench] the same workload with row_alignment={alt_ra} ...", file=sys.stderr, flush=True)
+        result["alt_layout"] = measure_alt_layout(args, dev, alt_ra, out_tensor(outs[0]))
     if not args.no_cpu_baseline:
         print("[bench] timing the CPU baseline ...", file=sys.stderr, flush=True)
         result["cpu_baseline"] = cpu_baseline(wl, out_tensor(outs[0]), args.cpu_seconds)
