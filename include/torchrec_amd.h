@@ -131,6 +131,33 @@ int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indi
                             int32_t pooling_mode, int32_t out_dtype, void* out,
                             int64_t out_stride, void* workspace, void* stream);
 
+/* Pooled lookup with position weights: the id at position k of a bag of the
+ * feature at key position p is weighted by
+ *   position_weights[key_start[p] + min(k, key_len[p] - 1)],  or 1 if key_len[p] == 0,
+ * inside the lookup kernel, in place of per_sample_weights.  Replaces the
+ * three steps of the reference's feature-processed collection:
+ * PositionWeightedModuleCollection.forward (fbgemm offsets_range + a gather per
+ * key, torchrec/modules/feature_processor_.py:193-260), the weighted KJT it
+ * builds (torchrec/modules/fp_embedding_modules.py:20-53) and the weighted TBE
+ * call (torchrec/quant/embedding_modules.py:547-557).
+ *   bags              device: offsets [num_keys*B + 1], or lengths [num_keys*B]
+ *                     when bags_are_lengths (workspace as for
+ *                     tra_tbe_forward_lengths, else NULL)
+ *   position_weights  device fp32 [position_weights_len >= 1], all keys' vectors
+ *   key_start/key_len HOST int32 [num_keys], checked against the table here
+ * A launch class (one weight type and lane width) may hold at most 128
+ * features (TRA_ERR_TOO_LARGE otherwise; the caller then materializes the
+ * weights with tra_position_weights and calls tra_tbe_forward).  Other
+ * arguments and the arithmetic as tra_tbe_forward; TRA_POOL_NONE is refused. */
+int tra_tbe_forward_position_weighted(tra_tbe_t tbe, const void* weights, const void* indices,
+                                      const void* bags, int32_t bags_are_lengths,
+                                      int32_t idx_is_i64, const float* position_weights,
+                                      int64_t position_weights_len, const int32_t* key_start,
+                                      const int32_t* key_len, int32_t num_keys,
+                                      int32_t batch_size, int64_t num_indices,
+                                      int32_t pooling_mode, int32_t out_dtype, void* out,
+                                      int64_t out_stride, void* workspace, void* stream);
+
 /* Which kernels a tra_tbe_forward with these sizes launches, one entry per
  * launch, "; "-separated, e.g. "tbe_pooled_cu_kernel dtype=int4 lane_bytes=8
  * slices=26".  lengths_num_keys > 0 asks about tra_tbe_forward_lengths with

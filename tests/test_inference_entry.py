@@ -305,3 +305,74 @@ def test_quant_fp_ebc_bit_exact_against_oracle():
                 psw[s:e] = t[: e - s]
     want = O.tbe_forward(O.pack_store(otables), [0, 1, 2], B, ids, offsets, psw, O.SUM, O.FP32)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,max_len,idt,from_offsets", [
+    (21, 10, torch.int32, False),      # small: static kernel
+    (33, 30, torch.int64, True),       # bags longer than the weight vectors (clamped), int64 ids, KJT with offsets
+    (4096, 40, torch.int32, False),    # window kernel, offsets derived inside the lookup kernel
+    (4096, 40, torch.int32, True),     # window kernel from offsets
+])
+def test_position_weights_inside_the_lookup_kernel(B, max_len, idt, from_offsets):
+    """The feature-processed collection looks the position weights up inside
+    the lookup kernel.  Same bits as materializing them first (the weights are
+    the same fp32 values either way), for a key order that differs from the
+    module's, a key without weights, an unused key, MEAN and SUM tables."""
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(B + max_len)
+    rows, D = 500, 64
+    names = ["a", "b", "c", "d"]
+    cfgs, quantized = [], {}
+    for t, name in enumerate(names):
+        q = torch.from_numpy(O.quantize_sbhalf(rng.normal(0, 0.1, (rows, D)).astype(np.float32), 4 if t % 2 else 8))
+        cfgs.append(EmbeddingBagConfig(name=f"t_{name}", embedding_dim=D, num_embeddings=rows, feature_names=[name],
+                                       data_type=DataType.INT4 if t % 2 else DataType.INT8,
+                                       pooling=PoolingType.MEAN if t == 3 and B < 1000 else PoolingType.SUM))
+        quantized[f"t_{name}"] = (q[:, :-4].to(dev), q[:, -4:].to(dev))
+    pw = PositionWeightedModuleCollection({"a": 20, "c": 7, "d": 20}, dev)  # "b" has none: weight 1
+    with torch.no_grad():
+        for p in pw.position_weights.values():
+            p.copy_(torch.rand_like(p) * 2 - 1)
+    m = QuantFPEBC(cfgs, True, dev, output_dtype=torch.half, table_name_to_quantized_weights=quantized,
+                   feature_processor=pw)
+    keys = ["c", "unused", "a", "d", "b"]
+    lengths = rng.integers(0, max_len + 1, len(keys) * B).astype(np.int64)
+    ids = rng.integers(0, rows, int(lengths.sum()))
+    kw = dict(keys=keys, values=torch.from_numpy(ids).to(idt).to(dev))
+    if from_offsets:
+        offsets = np.zeros(len(lengths) + 1, dtype=np.int64)
+        offsets[1:] = np.cumsum(lengths)
+        kjt = KeyedJaggedTensor(offsets=torch.from_numpy(offsets).to(idt).to(dev), **kw)
+    else:
+        kjt = KeyedJaggedTensor(lengths=torch.from_numpy(lengths).to(idt).to(dev), **kw)
+    fused = m(kjt)
+    materialized = QuantEBC.forward(m, pw(kjt))
+    assert fused.keys() == materialized.keys()
+    assert torch.equal(fused.values().view(torch.int16), materialized.values().view(torch.int16))
+    # a replaced weight vector is picked up
+    with torch.no_grad():
+        pw.position_weights["a"].mul_(0.5)
+    assert torch.equal(m(kjt).values().view(torch.int16), QuantEBC.forward(m, pw(kjt)).values().view(torch.int16))
+    assert not torch.equal(m(kjt).values(), fused.values())
+
+
+@pytest.mark.gpu
+def test_position_weighted_entry_checks_its_layout():
+    """The C entry point validates the host-side layout against the table."""
+    dev = torch.device("cuda:0")
+    rows, D, B = 50, 32, 4
+    q = torch.from_numpy(O.quantize_sbhalf(np.zeros((rows, D), dtype=np.float32), 8))
+    cfg = EmbeddingBagConfig(name="t", embedding_dim=D, num_embeddings=rows, feature_names=["f"], data_type=DataType.INT8)
+    m = QuantEBC([cfg], True, dev, table_name_to_quantized_weights={"t": (q[:, :-4].to(dev), q[:, -4:].to(dev))})
+    op = m._emb_modules[0]
+    ids = torch.zeros(8, dtype=torch.int32, device=dev)
+    offsets = torch.arange(0, 10, 2, dtype=torch.int32, device=dev)
+    table = torch.ones(6, device=dev)
+    op(ids, offsets, position_weights=(table, [0], [6]))
+    with pytest.raises(RuntimeError, match="outside the table"):
+        op(ids, offsets, position_weights=(table, [2], [6]))
+    with pytest.raises(RuntimeError, match="outside the table"):
+        op(ids, offsets, position_weights=(table, [-1], [3]))
+    with pytest.raises(AssertionError):
+        op(ids, offsets, position_weights=(table, [], []))

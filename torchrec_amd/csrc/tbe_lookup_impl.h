@@ -55,6 +55,13 @@ struct LookupArgs {
   int32_t out_fp16;
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
   int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
+  // Position weighting (posw != nullptr): the weight of the id at position k of
+  // a bag of class feature ci is posw[pw_off[ci] + min(k, pw_len[ci] - 1)], or
+  // 1 when pw_len[ci] is 0.  Takes the place of psw; classes of at most
+  // kMaxPos features.
+  const float* posw;
+  int32_t pw_off[kMaxPos];
+  int32_t pw_len[kMaxPos];
 #ifdef TRA_INSTRUMENT
   unsigned long long* ts;  // [waves][8] wall-clock stamps
 #endif
@@ -235,12 +242,33 @@ struct RowWalk {
   uint32_t row_bytes;
   int chunk_off;
   bool count_errors;
+  // position weighting: this bag's weight vector (always readable), its last
+  // index, whether the feature has one at all, and where the bag starts
+  const float* pw;
+  uint32_t pw_last;
+  bool pw_on;
+  int64_t bag_start;
+  __device__ __forceinline__ void set_position_weights(const LookupArgs& a, int ci, int64_t start);
   __device__ __forceinline__ void set_rows(int64_t r, int32_t rb) {
     rows = r;
     rows32 = r < (int64_t(1) << 31) ? (uint32_t)r : 0x80000000u;
     row_bytes = (uint32_t)rb;
   }
 };
+
+__device__ __forceinline__ void RowWalk::set_position_weights(const LookupArgs& a, int ci,
+                                                              int64_t start) {
+  pw = a.posw;
+  pw_last = 0;
+  pw_on = false;
+  bag_start = start;
+  if (a.posw != nullptr) {
+    const int n = ci < kMaxPos ? a.pw_len[ci] : 0;
+    pw_on = n > 0;
+    pw = a.posw + (n > 0 ? a.pw_off[ci] : 0);
+    pw_last = (uint32_t)(n > 0 ? n - 1 : 0);
+  }
+}
 
 // Id of position j, or -1 (= skip) when the position is outside the bag.  The
 // load itself is unconditional (position clamped into the ids array) and the
@@ -286,8 +314,17 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
   r.d = load_chunk<CB>(chunk);
   if constexpr (WEIGHTED) {
     using UIdxT = typename std::make_unsigned<IdxT>::type;
+    // One load either way: the per-sample weight of this id, or the position
+    // weight of its place in the bag, clamped into the feature's weight vector
+    // (a slot past the end of its bag reads some valid weight and is dropped
+    // later).  Selected by value, not by branch: the mode is a launch argument.
+    const bool by_position = a.posw != nullptr;
     const IdxT jc = (UIdxT)j < (UIdxT)last ? j : last;
-    r.w = a.psw[jc];
+    const UIdxT k = (UIdxT)(j - (IdxT)w.bag_start);
+    const uint32_t kc = k < (UIdxT)w.pw_last ? (uint32_t)k : w.pw_last;
+    const float* src = by_position ? w.pw + kc : a.psw + jc;
+    const float v = *src;
+    r.w = by_position && !w.pw_on ? 1.0f : v;
   } else {
     r.w = 1.0f;
   }
@@ -380,7 +417,7 @@ __device__ __forceinline__ int wave_max(int v) {
 
 // Locate this block's (sub-class, feature, tile).  Uniform across the block.
 __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lpr,
-                                            int& tile) {
+                                            int& tile, int* class_index = nullptr) {
   const int blk = blockIdx.x;
   int s = 0;
 #pragma unroll
@@ -392,6 +429,7 @@ __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lp
   if (fi >= sc.count) return false;
   tile = local - fi * sc.tiles_per_feat;
   f = a.feats[sc.first + fi];
+  if (class_index) *class_index = sc.first + fi;
   lpr = sc.lpr;
   return true;
 }
@@ -542,8 +580,8 @@ template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U>
 __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;  // columns per lane
   TRA_STAMP(0);
-  int f, lpr, tile;
-  if (!locate_tile(a, f, lpr, tile)) return;
+  int f, lpr, tile, ci;
+  if (!locate_tile(a, f, lpr, tile, &ci)) return;
   const FeatureDesc d = a.descs[f];
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int wave = threadIdx.x / kWaveSize;
@@ -568,6 +606,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
   w.lane_base = a.weights + d.table_offset + w.chunk_off;
   w.set_rows(d.rows, d.row_bytes);
   w.count_errors = c == 0 && d.payload_off == 0;
+  w.set_position_weights(a, ci, start);
 
   float acc[NE];
 #pragma unroll
@@ -878,6 +917,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     w.lane_base = a.weights + d.table_offset + w.chunk_off;
     w.set_rows(d.rows, d.row_bytes);
     w.count_errors = c == 0 && d.payload_off == 0;
+    w.set_position_weights(a, sc.first + fi, start);
 
     float acc[NE];
 #pragma unroll

@@ -323,11 +323,21 @@ int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
   return TRA_OK;
 }
 
+// Position weights of a call: one fp32 vector per input key, concatenated on
+// the device; key_start / key_len (host) say where key p's vector sits.
+struct PositionWeights {
+  const float* table;
+  int64_t table_len;
+  const int32_t* key_start;
+  const int32_t* key_len;
+  int32_t num_keys;
+};
+
 static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
                         const void* offsets, bool from_lengths, int32_t idx_is_i64,
                         const float* per_sample_weights, int32_t batch_size, int64_t num_indices,
                         int32_t pooling_mode, int32_t out_dtype, void* out, int64_t out_stride,
-                        void* stream) {
+                        void* stream, const PositionWeights* pw = nullptr) {
   if (!tbe) {
     set_error("tra_tbe_forward: null plan");
     return TRA_ERR_INVALID_ARGUMENT;
@@ -383,6 +393,31 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     a.offsets = offsets;
     // (no ids: nothing to weigh, and the weights pointer may not be readable)
     a.psw = nobag || num_indices == 0 ? nullptr : per_sample_weights;
+    if (pw != nullptr && !nobag && num_indices > 0) {
+      if (cls.feats.size() > (size_t)kMaxPos) {
+        set_error("position-weighted lookup: a launch class has %d features, at most %d are supported",
+                  (int)cls.feats.size(), kMaxPos);
+        return TRA_ERR_TOO_LARGE;
+      }
+      for (size_t i = 0; i < cls.feats.size(); ++i) {
+        const int key = tbe->slices[cls.feats[i]].feature;
+        if (key < 0 || key >= pw->num_keys) {
+          set_error("position-weighted lookup: feature at key position %d, but %d keys were described", key,
+                    pw->num_keys);
+          return TRA_ERR_INVALID_ARGUMENT;
+        }
+        const int64_t st = pw->key_start[key], n = pw->key_len[key];
+        if (n < 0 || st < 0 || (n > 0 && st + n > pw->table_len)) {
+          set_error("position-weighted lookup: key %d has weights [%lld, %lld) outside the table of %lld", key,
+                    (long long)st, (long long)(st + n), (long long)pw->table_len);
+          return TRA_ERR_INVALID_ARGUMENT;
+        }
+        a.pw_off[i] = (int32_t)st;
+        a.pw_len[i] = (int32_t)n;
+      }
+      a.posw = pw->table;
+      a.psw = nullptr;
+    }
     a.out = out;
     a.out_stride = out_stride;
     a.err_count = tbe->err_dev;
@@ -480,7 +515,7 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     }
     lp.unroll = tune.unroll;
     lp.idx64 = idx_is_i64 != 0;
-    lp.weighted = a.psw != nullptr;
+    lp.weighted = a.psw != nullptr || a.posw != nullptr;
     lp.nobag = nobag;
     lp.from_lengths = from_lengths;
     int rc;
@@ -512,11 +547,14 @@ int64_t tra_tbe_forward_lengths_workspace_bytes(int32_t num_keys, int32_t batch_
   return off_bytes + tra_cumsum_workspace_bytes(n);
 }
 
-int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indices,
-                            const void* lengths, int32_t idx_is_i64,
-                            const float* per_sample_weights, int32_t batch_size, int32_t num_keys,
-                            int64_t num_indices, int32_t pooling_mode, int32_t out_dtype, void* out,
-                            int64_t out_stride, void* workspace, void* stream) {
+}  // extern "C"
+
+static int forward_lengths_impl(tra_tbe_t tbe, const void* weights, const void* indices,
+                                const void* lengths, int32_t idx_is_i64,
+                                const float* per_sample_weights, int32_t batch_size,
+                                int32_t num_keys, int64_t num_indices, int32_t pooling_mode,
+                                int32_t out_dtype, void* out, int64_t out_stride, void* workspace,
+                                void* stream, const PositionWeights* pw) {
   if (!tbe) {
     set_error("tra_tbe_forward_lengths: null plan");
     return TRA_ERR_INVALID_ARGUMENT;
@@ -537,7 +575,7 @@ int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indi
   }
   if (fused_scan_possible(tbe, batch_size, num_keys, num_indices, pooling_mode, lengths))
     return forward_impl(tbe, weights, indices, lengths, true, idx_is_i64, per_sample_weights,
-                        batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream);
+                        batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream, pw);
   // Offsets first, then the ordinary lookup.
   const int64_t n = (int64_t)num_keys * batch_size;
   if (!workspace) {
@@ -550,7 +588,44 @@ int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indi
   const int rc = tra_cumsum(lengths, n, idx_is_i64, workspace, scan_ws, stream);
   if (rc != TRA_OK) return rc;
   return forward_impl(tbe, weights, indices, workspace, false, idx_is_i64, per_sample_weights,
-                      batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream);
+                      batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream, pw);
+}
+
+extern "C" {
+
+int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indices,
+                            const void* lengths, int32_t idx_is_i64,
+                            const float* per_sample_weights, int32_t batch_size, int32_t num_keys,
+                            int64_t num_indices, int32_t pooling_mode, int32_t out_dtype, void* out,
+                            int64_t out_stride, void* workspace, void* stream) {
+  return forward_lengths_impl(tbe, weights, indices, lengths, idx_is_i64, per_sample_weights,
+                              batch_size, num_keys, num_indices, pooling_mode, out_dtype, out,
+                              out_stride, workspace, stream, nullptr);
+}
+
+int tra_tbe_forward_position_weighted(tra_tbe_t tbe, const void* weights, const void* indices,
+                                      const void* bags, int32_t bags_are_lengths,
+                                      int32_t idx_is_i64, const float* position_weights,
+                                      int64_t position_weights_len, const int32_t* key_start,
+                                      const int32_t* key_len, int32_t num_keys, int32_t batch_size,
+                                      int64_t num_indices, int32_t pooling_mode, int32_t out_dtype,
+                                      void* out, int64_t out_stride, void* workspace,
+                                      void* stream) {
+  if (!position_weights || position_weights_len < 1 || !key_start || !key_len || num_keys < 0) {
+    set_error("tra_tbe_forward_position_weighted: null or empty position weight description");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (pooling_mode == TRA_POOL_NONE) {
+    set_error("tra_tbe_forward_position_weighted: position weights apply to pooled lookups only");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const PositionWeights pw{position_weights, position_weights_len, key_start, key_len, num_keys};
+  if (bags_are_lengths)
+    return forward_lengths_impl(tbe, weights, indices, bags, idx_is_i64, nullptr, batch_size,
+                                num_keys, num_indices, pooling_mode, out_dtype, out, out_stride,
+                                workspace, stream, &pw);
+  return forward_impl(tbe, weights, indices, bags, false, idx_is_i64, nullptr, batch_size,
+                      num_indices, pooling_mode, out_dtype, out, out_stride, stream, &pw);
 }
 
 int tra_tbe_error_count(tra_tbe_t tbe, void* stream, int64_t* count) {

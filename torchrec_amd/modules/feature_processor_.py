@@ -79,6 +79,7 @@ class PositionWeightedModuleCollection(FeatureProcessorsCollection, CopyMixIn):
             self.position_weights_dict[key] = self.position_weights[key]
         # (keys, device) -> (key_start, key_len) index tensors of the fused GPU path
         self._layout_cache: Dict[object, object] = {}
+        self._table_cache = None  # (stamp of the parameters, concatenated fp32 table)
         self.reset_parameters()
 
     def reset_parameters(self) -> None:
@@ -91,10 +92,12 @@ class PositionWeightedModuleCollection(FeatureProcessorsCollection, CopyMixIn):
         for k, p in self.position_weights.items():
             self.position_weights_dict[k] = p
         self._layout_cache = {}
+        self._table_cache = None
 
-    def _weights_gpu(self, features: KeyedJaggedTensor) -> torch.Tensor:
-        keys = features.keys()
-        dev = features.values().device
+    def _layout(self, keys: List[str], dev: torch.device):
+        """For a key order: where each key's weight vector sits in the
+        concatenation of the vectors of the keys that have one (start, length;
+        length 0 = weight 1), as host lists and as device tensors."""
         ck = (tuple(keys), dev)
         layout = self._layout_cache.get(ck)
         if layout is None:
@@ -111,16 +114,39 @@ class PositionWeightedModuleCollection(FeatureProcessorsCollection, CopyMixIn):
             layout = (
                 torch.tensor(starts, dtype=torch.int32, device=dev),
                 torch.tensor(lens, dtype=torch.int32, device=dev),
+                starts,
+                lens,
             )
             self._layout_cache[ck] = layout
+        return layout
+
+    def _table(self, keys: List[str], dev: torch.device) -> torch.Tensor:
+        """The weight vectors of ``keys`` in one fp32 tensor.  Rebuilt only when a
+        parameter was replaced or written to since the last call."""
         present = [self.position_weights_dict[k] for k in keys if k in self.position_weights_dict]
-        table = (
-            torch.cat([p.detach().float().to(dev) for p in present])
-            if present
-            else torch.zeros(1, dtype=torch.float32, device=dev)
-        )
+        stamp = (tuple(keys), dev, tuple((id(p), p._version) for p in present))
+        if self._table_cache is None or self._table_cache[0] != stamp:
+            table = (
+                torch.cat([p.detach().float().to(dev) for p in present])
+                if present
+                else torch.zeros(1, dtype=torch.float32, device=dev)
+            )
+            self._table_cache = (stamp, table)
+        return self._table_cache[1]
+
+    def kernel_layout(self, keys: List[str], dev: torch.device):
+        """``(table, key_start, key_len)`` as the lookup operator's
+        ``position_weights`` argument takes them."""
+        layout = self._layout(keys, dev)
+        return self._table(keys, dev), layout[2], layout[3]
+
+    def _weights_gpu(self, features: KeyedJaggedTensor) -> torch.Tensor:
+        keys = features.keys()
+        dev = features.values().device
+        layout = self._layout(keys, dev)
         return ops.position_weights(
-            features.offsets(), len(keys), features.stride(), layout[0], layout[1], table, features.values().numel()
+            features.offsets(), len(keys), features.stride(), layout[0], layout[1], self._table(keys, dev),
+            features.values().numel(),
         )
 
     def forward(self, features: KeyedJaggedTensor) -> KeyedJaggedTensor:

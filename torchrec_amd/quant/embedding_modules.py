@@ -49,7 +49,7 @@ from torchrec_amd.modules.embedding_modules import (
     EmbeddingCollectionInterface,
     get_embedding_names_by_table,
 )
-from torchrec_amd.modules.feature_processor_ import FeatureProcessorsCollection
+from torchrec_amd.modules.feature_processor_ import FeatureProcessorsCollection, PositionWeightedModuleCollection
 from torchrec_amd.modules.fp_embedding_modules import (
     FeatureProcessedEmbeddingBagCollection as OriginalFeatureProcessedEmbeddingBagCollection,
 )
@@ -436,8 +436,16 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
             self.tbes: torch.nn.ModuleList = torch.nn.ModuleList(self._emb_modules)
         setattr(self, MODULE_ATTR_CACHE_FEATURES_ORDER, cache_features_order)
 
-    def forward(self, features: KeyedJaggedTensor) -> KeyedTensor:
-        """``features``: KJT of shape [F x B x jagged] -> KeyedTensor [B, sum(dims)]."""
+    def forward(
+        self,
+        features: KeyedJaggedTensor,
+        position_weights: Optional[Tuple[Tensor, List[int], List[int]]] = None,
+    ) -> KeyedTensor:
+        """``features``: KJT of shape [F x B x jagged] -> KeyedTensor [B, sum(dims)].
+
+        ``position_weights`` (not an argument of the reference; the
+        feature-processed subclass passes it) weighs every id by its position
+        in its bag inside the lookup kernel, see the operator's ``forward``."""
         order = self._resolve_order(_get_kjt_keys(features))
         B = features.stride()
         indices = features.values()
@@ -454,7 +462,7 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
             offsets, lengths = None, features.lengths()
         else:
             offsets = features.offsets()
-        psw = features.weights() if self._is_weighted else None
+        psw = features.weights() if self._is_weighted and position_weights is None else None
         out = torch.empty((B, self._total_D), dtype=self._output_dtype, device=indices.device)
         col = 0
         for emb_op, positions in zip(self._emb_modules, self._group_positions(order)):
@@ -467,6 +475,7 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
                 batch_size=B,
                 out=out,
                 out_col=col,
+                position_weights=position_weights,
             )
             col += emb_op.total_D  # type: ignore[union-attr]
         return KeyedTensor(keys=self._embedding_names, values=out, length_per_key=self._length_per_key)
@@ -519,6 +528,11 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         return self._device
 
 
+# The lookup kernel keeps the position-weight layout of a launch in its launch
+# arguments: at most this many features per operator.
+_MAX_FUSED_POSITION_FEATURES = 128
+
+
 class FeatureProcessedEmbeddingBagCollection(EmbeddingBagCollection):
     """Quantized collection behind a feature processor
     (torchrec/quant/embedding_modules.py:633-731): ``forward`` first lets
@@ -554,8 +568,18 @@ class FeatureProcessedEmbeddingBagCollection(EmbeddingBagCollection):
         assert feature_processor is not None, "Use EmbeddingBagCollection for no feature_processor"
         self.feature_processor: FeatureProcessorsCollection = feature_processor
 
-    def forward(self, features: KeyedJaggedTensor) -> KeyedTensor:
-        return super().forward(self.feature_processor(features))
+    def forward(self, features: KeyedJaggedTensor) -> KeyedTensor:  # type: ignore[override]
+        # Position weights on the GPU are looked up inside the lookup kernel: no
+        # weight tensor is written and read back, and no weighted KJT is built.
+        fp = self.feature_processor
+        if (
+            isinstance(fp, PositionWeightedModuleCollection)
+            and features.values().device.type == "cuda"
+            and features.keys()
+            and all(len(op.feature_table_map) <= _MAX_FUSED_POSITION_FEATURES for op in self._emb_modules)
+        ):
+            return super().forward(features, position_weights=fp.kernel_layout(features.keys(), features.values().device))
+        return super().forward(fp(features))
 
     def _get_name(self) -> str:
         return "QuantFeatureProcessedEmbeddingBagCollection"

@@ -274,6 +274,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         out: Optional[Tensor] = None,
         out_col: int = 0,
         lengths: Optional[Tensor] = None,
+        position_weights: Optional[Tuple[Tensor, Sequence[int], Sequence[int]]] = None,
     ) -> Tensor:
         """Pooled: ``[B, total_D]``; ``PoolingMode.NONE``: ``[indices.numel(), D]``.
 
@@ -287,7 +288,11 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         (``[L, D]`` for PoolingMode.NONE).  With ``offsets=None`` and
         ``lengths`` (the KJT's ``[K * B]`` lengths, ``batch_size`` required) the
         operator derives the offsets itself, inside the lookup kernel when the
-        call is large enough for that to pay.
+        call is large enough for that to pay.  ``position_weights`` =
+        ``(table, key_start, key_len)`` replaces ``per_sample_weights`` by
+        weights looked up inside the kernel: the id at position ``k`` of a bag
+        of input key ``p`` gets ``table[key_start[p] + min(k, key_len[p] - 1)]``
+        (1 when ``key_len[p]`` is 0); ``table`` is one fp32 device tensor.
         """
         dev = self.current_device
         if dev.type != "cuda":
@@ -336,6 +341,18 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         out_dtype = torch.float16 if self.output_dtype == _lib.FP16 else torch.float32
         nobag = self.pooling_mode == PoolingMode.NONE
         psw = None
+        pos_args = None
+        if position_weights is not None:
+            assert not nobag, "position weights apply to pooled lookups"
+            assert per_sample_weights is None, "position weights take the place of per_sample_weights"
+            table, key_start, key_len = position_weights
+            _lib.require_gpu(table, "position weight table")
+            assert table.dtype == torch.float32 and table.is_contiguous() and table.numel() >= 1
+            n_k = len(key_start)
+            assert len(key_len) == n_k >= n_keys, "one (start, length) pair per input key"
+            pos_args = (
+                table, (ctypes.c_int32 * max(n_k, 1))(*key_start), (ctypes.c_int32 * max(n_k, 1))(*key_len), n_k
+            )
         if per_sample_weights is not None and not nobag:
             psw = per_sample_weights.contiguous()
             if psw.dtype != torch.float32:
@@ -354,7 +371,26 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         out_stride = out.stride(0)
         out_ptr = out.data_ptr() + out_col * out.element_size()
         i64 = int(indices.dtype == torch.int64)
-        if offsets is None:
+        if pos_args is not None:
+            table, c_start, c_len, n_k = pos_args
+            stream = _lib.current_stream(dev)
+            ws_ptr = None
+            if offsets is None:
+                assert k_total == n_k, "one (start, length) pair per key of the lengths"
+                ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
+                ws = self._workspace.get(stream)
+                if ws is None or ws.numel() < ws_bytes or ws.device != dev:
+                    ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+                ws_ptr = ws.data_ptr()
+            _lib.check(
+                _lib.lib().tra_tbe_forward_position_weighted(
+                    self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices),
+                    _lib.ptr(lengths if offsets is None else offsets), int(offsets is None), i64,
+                    _lib.ptr(table), table.numel(), c_start, c_len, n_k, B, L, int(self.pooling_mode),
+                    self.output_dtype, out_ptr, out_stride, ws_ptr, stream,
+                )
+            )
+        elif offsets is None:
             ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
             stream = _lib.current_stream(dev)
             # one scratch buffer per stream: calls queued on different streams must not share it
