@@ -284,12 +284,17 @@ __device__ __forceinline__ IdxT fetch_id(const LookupArgs& a, bool in_range, Idx
   return in_range ? id : (IdxT)-1;
 }
 
+// Values of the kernels' WEIGHTED parameter: how a row's weight is obtained.
+constexpr int kUnweighted = 0;
+constexpr int kPerSample = 1;   // psw[j]
+constexpr int kByPosition = 2;  // position weight of the id's place in its bag
+
 // Issue the loads of one row chunk (header dword, CB payload bytes, weight).
 // Branch-free: an id outside [0, rows) (a pruned id -1, a lane past the end of
 // its bag, or a bad id) is redirected to row 0 and flagged invalid; consume_row
 // then multiplies it away exactly.  Returns 1 for a bad id (out of range and
 // not -1).
-template <int DTYPE, int CB, bool WEIGHTED, typename IdxT>
+template <int DTYPE, int CB, int WEIGHTED, typename IdxT>
 __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT last,
                                           const LookupArgs& a, const RowWalk& w) {
   const uint8_t* lane_base = w.lane_base;  // table + this lane's chunk offset
@@ -314,17 +319,18 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
   r.d = load_chunk<CB>(chunk);
   if constexpr (WEIGHTED) {
     using UIdxT = typename std::make_unsigned<IdxT>::type;
-    // One load either way: the per-sample weight of this id, or the position
-    // weight of its place in the bag, clamped into the feature's weight vector
-    // (a slot past the end of its bag reads some valid weight and is dropped
-    // later).  Selected by value, not by branch: the mode is a launch argument.
-    const bool by_position = a.posw != nullptr;
-    const IdxT jc = (UIdxT)j < (UIdxT)last ? j : last;
-    const UIdxT k = (UIdxT)(j - (IdxT)w.bag_start);
-    const uint32_t kc = k < (UIdxT)w.pw_last ? (uint32_t)k : w.pw_last;
-    const float* src = by_position ? w.pw + kc : a.psw + jc;
-    const float v = *src;
-    r.w = by_position && !w.pw_on ? 1.0f : v;
+    if constexpr (WEIGHTED == kByPosition) {
+      // The weight of this id's place in its bag, clamped into the feature's
+      // weight vector (a slot past the end of its bag reads some valid weight
+      // and is dropped later); 1 for a feature without position weights.
+      const UIdxT k = (UIdxT)(j - (IdxT)w.bag_start);
+      const uint32_t kc = k < (UIdxT)w.pw_last ? (uint32_t)k : w.pw_last;
+      const float v = w.pw[kc];
+      r.w = w.pw_on ? v : 1.0f;
+    } else {
+      const IdxT jc = (UIdxT)j < (UIdxT)last ? j : last;
+      r.w = a.psw[jc];
+    }
   } else {
     r.w = 1.0f;
   }
@@ -454,7 +460,7 @@ __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lp
 // count).  Software pipeline, per lane group: ids are requested two batches of
 // U rows ahead, row chunks one batch ahead, so neither an id load nor a row
 // load is waited for in the batch that issued it.
-template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, int NE>
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, int NE>
 __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
                                          const RowWalk& w, int64_t start64, int len,
                                          int max_len_any_lane) {
@@ -484,7 +490,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], idB[u], start + it + U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufA[u]);
+      if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u]);
     if (it + U >= max_len) break;
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -494,7 +500,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], idA[u], start + it + 2 * U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + U + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
+      if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u]);
   }
   // Bad ids are counted by the lane that owns column 0.
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
@@ -506,7 +512,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
 // lpr rows instead of one per row.  Needs lpr >= 2*U (a power of two): the
 // block after the current one, requested when the current one is entered, is
 // then at least two batches ahead, like the ids of pool_bag.
-template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, int NE>
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, int NE>
 __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs& a,
                                               const RowWalk& w, int64_t start64, int len,
                                               int max_len_any_lane, int lpr, int c,
@@ -550,7 +556,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufA[u]);
+      if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u]);
     if (it + U >= max_len) break;
     enter(it + 2 * U);
 #pragma unroll
@@ -558,7 +564,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + U + u < max_len) consume_row<DTYPE, CB, WEIGHTED>(acc, bufB[u]);
+      if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u]);
   }
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
 }
@@ -576,7 +582,7 @@ __device__ __forceinline__ void finish_bag(float (&acc)[NE], const LookupArgs& a
 
 // Static mapping: lane group g of wave w of tile t owns bag (t*waves + w)*gpw + g.
 // Used for small problems, where there are not enough bags to balance.
-template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U>
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U>
 __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;  // columns per lane
   TRA_STAMP(0);
@@ -705,7 +711,7 @@ __device__ __forceinline__ int feat_key_pos(const LookupArgs& a, const SubClass&
 // FROM_LENGTHS: a.offsets points at the KJT's lengths instead of its offsets
 // and the block derives its bags' start positions itself: one block-wide sum
 // of everything in front of the window plus a scan of the window in LDS.
-template <int DTYPE, int CB, typename IdxT, bool WEIGHTED, int U, bool FROM_LENGTHS = false>
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, bool FROM_LENGTHS = false>
 __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;
   extern __shared__ unsigned char tra_dyn_smem[];  // only its size matters (one block per CU)
@@ -1024,10 +1030,12 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
       hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kBlockThreads), 0, \
                          stream, a);                                                           \
   } while (0)
-  if (p.weighted) {
-    if (p.unroll >= 8) TRA_POOLED(true, 8); else if (p.unroll >= 4) TRA_POOLED(true, 4); else TRA_POOLED(true, 2);
+  if (a.posw != nullptr) {
+    TRA_POOLED(kByPosition, 4);  // (one unroll depth: the others are tuning variants)
+  } else if (p.weighted) {
+    if (p.unroll >= 8) TRA_POOLED(kPerSample, 8); else if (p.unroll >= 4) TRA_POOLED(kPerSample, 4); else TRA_POOLED(kPerSample, 2);
   } else {
-    if (p.unroll >= 8) TRA_POOLED(false, 8); else if (p.unroll >= 4) TRA_POOLED(false, 4); else TRA_POOLED(false, 2);
+    if (p.unroll >= 8) TRA_POOLED(kUnweighted, 8); else if (p.unroll >= 4) TRA_POOLED(kUnweighted, 4); else TRA_POOLED(kUnweighted, 2);
   }
 #undef TRA_POOLED
 }
