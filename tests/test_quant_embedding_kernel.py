@@ -327,3 +327,39 @@ def test_from_float_module():
             lo, hi = offs[f * 16 + b], offs[f * 16 + b + 1]
             want[b, f * 32:(f + 1) * 32] = w.detach().cpu()[ids[lo:hi]].sum(dim=0)
     torch.testing.assert_close(got.cpu(), want, atol=0.1, rtol=0)
+
+
+def _unwrap_case(offsets_dtype, indices_dtype, device):
+    """torchrec/quant/tests/test_embedding_modules.py:999-1025: the unsharded and
+    the per-shard modules hand the operator the same dtypes."""
+    from torchrec_amd.distributed.quant_embedding_kernel import _unwrap_kjt, _unwrap_kjt_for_cpu
+    from torchrec_amd.quant.embedding_modules import _fx_trec_unwrap_kjt
+
+    features = KeyedJaggedTensor(
+        keys=["f1", "f2", "f3", "f4"],
+        values=torch.tensor([0, 1, 2, 3, 4, 5, 6, 7], dtype=indices_dtype, device=device),
+        offsets=torch.tensor([0, 2, 5, 7, 8], dtype=offsets_dtype, device=device),
+    )
+    indices, offsets = _fx_trec_unwrap_kjt(features)
+    assert indices.dtype == offsets.dtype
+    if device.type == "cpu":
+        sharded_indices, sharded_offsets, _ = _unwrap_kjt_for_cpu(features, weighted=False)
+        assert sharded_indices.dtype == indices_dtype
+    else:
+        sharded_indices, sharded_offsets, _ = _unwrap_kjt(features)
+        assert sharded_indices.dtype == torch.int32
+    assert indices.dtype == sharded_indices.dtype and offsets.dtype == sharded_offsets.dtype
+    assert torch.equal(indices, sharded_indices) and torch.equal(offsets, sharded_offsets)
+
+
+@pytest.mark.parametrize("offsets_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("indices_dtype", [torch.int32, torch.int64])
+def test_unwrap_unsharded_vs_per_shard_in_sync_host(offsets_dtype, indices_dtype):
+    _unwrap_case(offsets_dtype, indices_dtype, torch.device("cpu"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("offsets_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("indices_dtype", [torch.int32, torch.int64])
+def test_unwrap_unsharded_vs_per_shard_in_sync_device(offsets_dtype, indices_dtype):
+    _unwrap_case(offsets_dtype, indices_dtype, torch.device("cuda:0"))

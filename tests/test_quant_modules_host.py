@@ -164,3 +164,16 @@ def test_feature_order_is_resolved_per_key_order():
     pinned = QuantEBC(tables, False, CPU, cache_features_order=True)
     first = pinned._resolve_order(["f3", "f2", "f1"])
     assert first == [2, 0, 1] and pinned._resolve_order(["f1", "f2", "f3"]) is first
+
+
+def test_create_on_meta_device_without_providing_weights():
+    """torchrec/quant/tests/test_embedding_modules.py:220-236."""
+    from torchrec_amd.modules.embedding_configs import EmbeddingBagConfig, EmbeddingConfig
+    from torchrec_amd.quant import EmbeddingBagCollection as QEBC, EmbeddingCollection as QEC
+
+    qebc = QEBC([EmbeddingBagConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1"])],
+                is_weighted=False, device=torch.device("meta"))
+    assert qebc.state_dict()["embedding_bags.t1.weight"].device.type == "meta"
+    qec = QEC([EmbeddingConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1"])],
+              device=torch.device("meta"))
+    assert qec.state_dict()["embeddings.t1.weight"].device.type == "meta"

@@ -528,12 +528,14 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
   IdxT cur = load_block(0);
   IdxT nxt = load_block(1);
   int cur_j = 0;
-  // Id of row r (wave-uniform r inside block cur_j or cur_j + 1), or -1 past the bag's end.
+  // Id of row r (wave-uniform), or -1 past the bag's end.  r lies in the
+  // current block: a batch of U rows never straddles two blocks (U divides
+  // lpr) and enter() is called before each batch.  Reading `cur` only matters:
+  // a select between cur and nxt would wait for the load of nxt that enter()
+  // has just issued.
   auto id_of = [&](int r) -> IdxT {
-    const int j = r / lpr_u;
-    const int src = group_lane0 + (r - j * lpr_u);
-    const IdxT v = j == cur_j ? cur : nxt;
-    return (IdxT)__shfl(v, src, kWaveSize);
+    const int src = group_lane0 + (r - cur_j * lpr_u);
+    return (IdxT)__shfl(cur, src, kWaveSize);
   };
   // Entering the block of row rb: make it the current one and request the next.
   auto enter = [&](int rb) {
