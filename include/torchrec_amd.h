@@ -275,6 +275,17 @@ int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys,
 int tra_mch_remap(const void* values, int64_t n, int32_t is_i64,
                   const int64_t* sorted_ids, const int64_t* mapping,
                   int64_t table_size, int64_t miss_id, void* out, void* stream);
+/* The same remap for all keys of a KeyedJaggedTensor in one launch: key k's
+ * ids are values[offsets[k*B] .. offsets[(k+1)*B]) (offsets: device
+ * [num_keys*B + 1], same integer type as values) and are looked up in key k's
+ * own table.  sorted_ids / mapping: HOST arrays of num_keys device pointers;
+ * table_size / miss_id: HOST arrays.  Replaces the per-table loop of
+ * ManagedCollisionCollection.forward (KJT split, one remap per table, cat;
+ * torchrec/modules/mc_modules.py:383-430). */
+int tra_mch_remap_keys(const void* values, int64_t n, const void* offsets, int32_t is_i64,
+                       int32_t num_keys, int32_t batch_size, const int64_t* const* sorted_ids,
+                       const int64_t* const* mapping, const int64_t* table_size,
+                       const int64_t* miss_id, void* out, void* stream);
 
 /* Measurement ------------------------------------------------------------- */
 /* Streaming device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte

@@ -116,3 +116,51 @@ def test_quant_mcec_matches_float():
     for k in ("f1", "f2", "f3"):
         assert torch.equal(got[k].lengths(), want[k].lengths())
         assert torch.allclose(got[k].values(), want[k].values(), atol=2e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+def test_collection_remaps_all_keys_in_one_launch(idt):
+    """The collection's GPU path (every key in one launch) against numpy's
+    searchsorted per table: two features on one table, one key without ids, a
+    key order that differs from the tables'."""
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(11)
+    sizes = {"t1": (500, 300), "t2": (64, 63), "t3": (2000, 1500)}
+    configs = [EmbeddingConfig(name="t1", embedding_dim=8, num_embeddings=500, feature_names=["a", "b"]),
+               EmbeddingConfig(name="t2", embedding_dim=8, num_embeddings=64, feature_names=["c"]),
+               EmbeddingConfig(name="t3", embedding_dim=8, num_embeddings=2000, feature_names=["d"])]
+    modules, tables = {}, {}
+    for name, (size, filled) in sizes.items():
+        raw = rng.choice(2**31 - 2, filled, replace=False).astype(np.int64)
+        rows = rng.permutation(size - 1)[:filled].astype(np.int64)
+        mod = MCHManagedCollisionModule(size, dev)
+        mod.set_id_table(torch.from_numpy(raw), torch.from_numpy(rows))
+        modules[name] = mod
+        tables[name] = (raw, rows, size - 1)
+    mcc = ManagedCollisionCollection(modules, configs).eval()
+    keys, B = ["d", "a", "c", "b"], 19
+    lengths = rng.integers(0, 9, len(keys) * B)
+    lengths[2 * B:3 * B] = 0  # "c" has no ids at all
+    table_of = {"a": "t1", "b": "t1", "c": "t2", "d": "t3"}
+    vals = []
+    for k, key in enumerate(keys):
+        raw = tables[table_of[key]][0]
+        n = int(lengths[k * B:(k + 1) * B].sum())
+        known = rng.choice(raw, n)
+        unknown = rng.integers(0, 2**31 - 2, n)
+        vals.append(np.where(rng.random(n) < 0.6, known, unknown))
+    values = np.concatenate(vals).astype(np.int64)
+    kjt = KeyedJaggedTensor(keys=keys, values=torch.from_numpy(values).to(idt).to(dev),
+                            lengths=torch.from_numpy(lengths).to(dev))
+    out = mcc(kjt)
+    assert out.keys() == ["a", "b", "c", "d"] and out.values().dtype == idt
+    per_key = dict(zip(keys, vals))
+    want = []
+    for key in out.keys():
+        raw, rows, miss = tables[table_of[key]]
+        lut = dict(zip(raw.tolist(), rows.tolist()))
+        want += [lut.get(int(v), miss) for v in per_key[key]]
+    assert out.values().cpu().tolist() == want
+    assert out.lengths().cpu().tolist() == np.concatenate(
+        [lengths[keys.index(k) * B:(keys.index(k) + 1) * B] for k in out.keys()]).tolist()

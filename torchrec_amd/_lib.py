@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = [
     "tra_offsets_range",
     "tra_position_weights",
     "tra_mch_remap",
+    "tra_mch_remap_keys",
     "tra_copy_bytes",
 ]
 
@@ -106,6 +107,10 @@ def lib() -> ctypes.CDLL:
         l.tra_offsets_range.argtypes = [vp, i64, i32, i64, vp, vp]
         l.tra_position_weights.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp]
         l.tra_mch_remap.argtypes = [vp, i64, i32, vp, vp, i64, i64, vp, vp]
+        l.tra_mch_remap_keys.argtypes = [
+            vp, i64, vp, i32, i32, i32, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64),
+            ctypes.POINTER(i64), vp, vp,
+        ]
         l.tra_copy_bytes.argtypes = [vp, vp, i64, vp]
         _lib = l
     return _lib

@@ -4,6 +4,7 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <cstring>
 
 #include "tra_common.h"
 
@@ -366,6 +367,41 @@ __global__ void mch_remap_kernel(const void* values, int64_t n, const int64_t* s
   }
 }
 
+// The same remap for every key of a KJT in one launch: blockIdx.y is the key,
+// its ids are values[offsets[key*B] .. offsets[(key+1)*B]) and it has its own
+// sorted table.  Tables travel in the launch arguments, kRemapKeys per launch.
+constexpr int kRemapKeys = 64;
+struct RemapTables {
+  const int64_t* sorted_ids[kRemapKeys];
+  const int64_t* mapping[kRemapKeys];
+  int64_t size[kRemapKeys];
+  int64_t miss_id[kRemapKeys];
+  int32_t first_key;  // key of blockIdx.y == 0
+};
+
+template <typename T>
+__global__ void mch_remap_keys_kernel(const void* values, int64_t n, const void* offsets, int32_t B,
+                                      const RemapTables t, void* out) {
+  const int k = blockIdx.y;
+  const int64_t key = (int64_t)t.first_key + k;
+  int64_t first = ld<T>(offsets, key * B), last = ld<T>(offsets, (key + 1) * B);
+  first = first < 0 ? 0 : first;
+  last = last > n ? n : last;
+  const int64_t* sorted_ids = t.sorted_ids[k];
+  const int64_t* mapping = t.mapping[k];
+  const int64_t size = t.size[k], miss_id = t.miss_id[k];
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t j = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < last; j += stride) {
+    const int64_t v = ld<T>(values, j);
+    int64_t lo = 0, hi = size - 1;
+    while (lo < hi) {
+      const int64_t mid = lo + ((hi - lo) >> 1);
+      if (sorted_ids[mid] < v) lo = mid + 1; else hi = mid;
+    }
+    st<T>(out, j, sorted_ids[lo] == v ? mapping[lo] : miss_id);
+  }
+}
+
 // Plain streaming copy, 16 bytes per lane per step.
 __global__ __launch_bounds__(256) void tra_copy_kernel(const uint4* __restrict__ src,
                                                         uint4* __restrict__ dst, int64_t n16) {
@@ -679,6 +715,50 @@ int tra_mch_remap(const void* values, int64_t n, int32_t is_i64, const int64_t* 
     hipLaunchKernelGGL(mch_remap_kernel<int32_t>, dim3(grid), dim3(256), 0, (hipStream_t)stream, values,
                        n, sorted_ids, mapping, table_size, miss_id, out);
   return check_launch("tra_mch_remap");
+}
+
+int tra_mch_remap_keys(const void* values, int64_t n, const void* offsets, int32_t is_i64,
+                       int32_t num_keys, int32_t batch_size, const int64_t* const* sorted_ids,
+                       const int64_t* const* mapping, const int64_t* table_size,
+                       const int64_t* miss_id, void* out, void* stream) {
+  if (n < 0 || num_keys < 0 || batch_size < 0) {
+    set_error("tra_mch_remap_keys: negative size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (n == 0 || num_keys == 0) return TRA_OK;
+  if (!values || !offsets || !out || !sorted_ids || !mapping || !table_size || !miss_id) {
+    set_error("tra_mch_remap_keys: null argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  for (int k = 0; k < num_keys; ++k)
+    if (!sorted_ids[k] || !mapping[k] || table_size[k] < 1) {
+      set_error("tra_mch_remap_keys: key %d has no table", k);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+  // blocks per key: enough for the average key, at most 1024
+  const int64_t per_key = n / num_keys + 1;
+  const unsigned gx = (unsigned)std::max<int64_t>(1, std::min<int64_t>((per_key + 255) / 256, 1024));
+  for (int k0 = 0; k0 < num_keys; k0 += kRemapKeys) {
+    const int nk = std::min(kRemapKeys, num_keys - k0);
+    RemapTables t;
+    std::memset(&t, 0, sizeof(t));
+    for (int k = 0; k < nk; ++k) {
+      t.sorted_ids[k] = sorted_ids[k0 + k];
+      t.mapping[k] = mapping[k0 + k];
+      t.size[k] = table_size[k0 + k];
+      t.miss_id[k] = miss_id[k0 + k];
+    }
+    t.first_key = k0;
+    if (is_i64)
+      hipLaunchKernelGGL(mch_remap_keys_kernel<int64_t>, dim3(gx, nk), dim3(256), 0, (hipStream_t)stream,
+                         values, n, offsets, batch_size, t, out);
+    else
+      hipLaunchKernelGGL(mch_remap_keys_kernel<int32_t>, dim3(gx, nk), dim3(256), 0, (hipStream_t)stream,
+                         values, n, offsets, batch_size, t, out);
+    const int rc = check_launch("tra_mch_remap_keys");
+    if (rc != TRA_OK) return rc;
+  }
+  return TRA_OK;
 }
 
 int tra_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream) {

@@ -179,10 +179,44 @@ class ManagedCollisionCollection(nn.Module):
     def embedding_configs(self) -> Sequence[BaseEmbeddingConfig]:
         return self._embedding_configs
 
+    def _one_launch_tables(self, features: KeyedJaggedTensor):
+        """Per key of ``features`` (already in table order) the sorted-id table, row
+        mapping and miss row of its module, when every module is an inference-mode
+        MCH module without an input hash and the ids are on the GPU; else None."""
+        if features.values().device.type != "cuda" or not features.keys():
+            return None
+        sorted_ids, mappings, miss = [], [], []
+        for config in self._embedding_configs:
+            module = self._managed_collision_modules[config.name]
+            if (
+                type(module) is not MCHManagedCollisionModule
+                or module.training
+                or module._input_hash_func is not None
+                or module._mch_sorted_raw_ids.device != features.values().device
+            ):
+                return None
+            for _ in config.feature_names:
+                sorted_ids.append(module._mch_sorted_raw_ids)
+                mappings.append(module._mch_remapped_ids_mapping)
+                miss.append(module._output_global_offset + module._zch_size - 1)
+        return sorted_ids, mappings, miss
+
     def forward(self, features: KeyedJaggedTensor) -> KeyedJaggedTensor:
         order = [features.keys().index(f) for f in self._feature_names]
         if order != list(range(len(features.keys()))):
             features = features.permute(order)
+        tables = self._one_launch_tables(features)
+        if tables is not None:
+            # all keys in one launch: no split per table, no host read of the
+            # per-key id counts, no concatenation
+            return KeyedJaggedTensor(
+                keys=features.keys(),
+                values=ops.mch_remap_keys(features.values(), features.offsets(), features.stride(), *tables),
+                lengths=features.lengths(),
+                offsets=features.offsets(),
+                weights=features.weights_or_none(),
+                stride=features.stride(),
+            )
         splits = features.split(self._table_feature_splits)
         values: List[torch.Tensor] = []
         # modules are visited in table (config) order, which is the order of the splits

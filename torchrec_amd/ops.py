@@ -309,3 +309,40 @@ def mch_remap(
         )
     )
     return out
+
+
+def mch_remap_keys(
+    values: torch.Tensor,
+    offsets: torch.Tensor,
+    batch_size: int,
+    sorted_ids: List[torch.Tensor],
+    mappings: List[torch.Tensor],
+    miss_ids: List[int],
+) -> torch.Tensor:
+    """``mch_remap`` for every key of a KeyedJaggedTensor in one launch: key ``k`` (ids
+    ``values[offsets[k*B] : offsets[(k+1)*B]]``) is looked up in ``sorted_ids[k]`` / ``mappings[k]``."""
+    import ctypes
+
+    _lib.require_gpu(values, "mch_remap_keys")
+    _check_int(values, "values")
+    K = len(sorted_ids)
+    assert len(mappings) == K and len(miss_ids) == K
+    assert offsets.numel() == K * batch_size + 1, "offsets must have num_keys * B + 1 entries"
+    for s_, m_ in zip(sorted_ids, mappings):
+        assert s_.dtype == torch.int64 and m_.dtype == torch.int64 and s_.numel() == m_.numel() > 0
+        assert s_.is_contiguous() and m_.is_contiguous() and s_.device == values.device and m_.device == values.device
+    values = values.contiguous()
+    if offsets.dtype != values.dtype:
+        offsets = offsets.to(values.dtype)
+    offsets = offsets.contiguous()
+    out = torch.empty_like(values)
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+    _lib.check(
+        _lib.lib().tra_mch_remap_keys(
+            _lib.ptr(values), values.numel(), _lib.ptr(offsets), int(values.dtype == torch.int64), K, int(batch_size),
+            (vp * max(K, 1))(*[t.data_ptr() for t in sorted_ids]), (vp * max(K, 1))(*[t.data_ptr() for t in mappings]),
+            (i64 * max(K, 1))(*[t.numel() for t in sorted_ids]), (i64 * max(K, 1))(*[int(m) for m in miss_ids]),
+            _lib.ptr(out), _lib.current_stream(values.device),
+        )
+    )
+    return out
