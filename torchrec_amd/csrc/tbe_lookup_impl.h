@@ -660,47 +660,108 @@ struct SumOf { using type = int64_t; };
 template <>
 struct SumOf<int32_t> { using type = int32_t; };
 
-// This thread's share of sum(lengths[0 .. p)): the block reads the range 16
-// bytes per lane per step, eight independent loads at a time (indices past the
-// end are clamped and their values dropped, so no load is predicated).  Every
-// block of the grid reads a prefix of the same array at the same moment, so
-// each starts at a different 16 KB step (`rot`) to spread the L2 channels.
+// This thread's share of sum(lengths[0 .. p)).  The block reads the range 16
+// bytes per lane per step, kPrefixBatch independent loads at a time (a lane's
+// index past the end is clamped and its value dropped, so no load is
+// predicated per lane; steps past the end are skipped for the whole wave).
+// start() adds up every batch but the last and leaves the last one in flight;
+// finish() adds it, so the last round trip overlaps whatever the caller does
+// between the two calls.
+// Every block of the grid reads a prefix of the same array at the same moment,
+// so each starts at a different 16 KB step (`rot`) to spread the L2 channels.
 // `lengths` is 16-byte aligned.
-template <typename IdxT>
-__device__ __forceinline__ typename SumOf<IdxT>::type prefix_partial(const IdxT* __restrict__ lengths,
-                                                                     int64_t p, int rot) {
-  using S = typename SumOf<IdxT>::type;
-  constexpr int V = 16 / (int)sizeof(IdxT);
-  struct __align__(16) Vec { IdxT v[V]; };
-  const Vec* vin = reinterpret_cast<const Vec*>(lengths);
-  const int nvec = (int)(p / V);
-  const int nk = (nvec + kCuThreads - 1) / kCuThreads;
-  S part = 0;
-  for (int k0 = 0; k0 < nk; k0 += 8) {
-    Vec x[8];
-    int idx[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      idx[k] = ((k0 + k + rot) % nk) * kCuThreads + (int)threadIdx.x;
-      x[k] = vin[min(idx[k], nvec - 1)];
-    }
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      S sum = 0;
-#pragma unroll
-      for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
-      part += (k0 + k < nk && idx[k] < nvec) ? sum : (S)0;
-    }
-  }
-  if ((int64_t)threadIdx.x < p - (int64_t)nvec * V) part += (S)lengths[(int64_t)nvec * V + threadIdx.x];
-  return part;
-}
+constexpr int kPrefixBatch = 8;
 
-template <typename S>
-__device__ __forceinline__ S wave_total_t(S v) {
+template <typename IdxT>
+struct PrefixSum {
+  using S = typename SumOf<IdxT>::type;
+  static constexpr int V = 16 / (int)sizeof(IdxT);
+  struct __align__(16) Vec { IdxT v[V]; };
+
+  const Vec* vin;
+  int nvec, nk, rot, k_last;
+  S part;
+  IdxT tail;
+  Vec x[kPrefixBatch];
+
+  // step k of this block's rotated order (k < nk, rot < nk: one wrap at most)
+  __device__ __forceinline__ int index_of(int k) const {
+    const int j = k + rot;
+    return (j >= nk ? j - nk : j) * kCuThreads + (int)threadIdx.x;
+  }
+  __device__ __forceinline__ void issue(int k0) {
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWaveSize);
+    for (int k = 0; k < kPrefixBatch; ++k)
+      if (k0 + k < nk) x[k] = vin[min(index_of(k0 + k), nvec - 1)];
+  }
+  __device__ __forceinline__ void consume(int k0) {
+#pragma unroll
+    for (int k = 0; k < kPrefixBatch; ++k)
+      if (k0 + k < nk) {
+        S sum = 0;
+#pragma unroll
+        for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
+        part += index_of(k0 + k) < nvec ? sum : (S)0;
+      }
+  }
+  __device__ __forceinline__ void start(const IdxT* __restrict__ lengths, int64_t p, int rot_) {
+    vin = reinterpret_cast<const Vec*>(lengths);
+    nvec = (int)(p / V);
+    nk = (nvec + kCuThreads - 1) / kCuThreads;
+    rot = nk > 0 ? rot_ % nk : 0;
+    part = 0;
+    // the elements after the last whole 16-byte step: one per lane, clamped like the rest
+    const int64_t rest = p - (int64_t)nvec * V;
+    const int64_t ti = (int64_t)nvec * V + min((int64_t)threadIdx.x, max(rest - 1, (int64_t)0));
+    tail = lengths[max(min(ti, p - 1), (int64_t)0)];
+    if ((int64_t)threadIdx.x >= rest) tail = 0;
+    k_last = nk > 0 ? ((nk - 1) / kPrefixBatch) * kPrefixBatch : 0;
+    for (int k0 = 0; k0 < k_last; k0 += kPrefixBatch) {
+      issue(k0);
+      consume(k0);
+    }
+    issue(k_last);
+  }
+  __device__ __forceinline__ S finish() {
+    consume(k_last);
+    return part + (S)tail;
+  }
+};
+
+// Inclusive scan over the 64 lanes of a wave.  32-bit sums use the data-parallel
+// lane moves of the VALU (shifts inside each row of 16 lanes, then lane 15 and
+// lane 31 broadcast into the following rows): six adds, no trip through the LDS
+// crossbar.  Lanes without a source receive 0.
+__device__ __forceinline__ int32_t wave_scan_incl(int32_t v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
   return v;
+}
+__device__ __forceinline__ int64_t wave_scan_incl(int64_t v) {
+  const int ln = threadIdx.x & (kWaveSize - 1);
+#pragma unroll
+  for (int off = 1; off < kWaveSize; off <<= 1) {
+    const int64_t o = __shfl_up(v, off, kWaveSize);
+    if (ln >= off) v += o;
+  }
+  return v;
+}
+// Lane 63's value of v, in every lane.
+__device__ __forceinline__ int32_t wave_last(int32_t v) { return __builtin_amdgcn_readlane(v, kWaveSize - 1); }
+__device__ __forceinline__ int64_t wave_last(int64_t v) { return __shfl(v, kWaveSize - 1, kWaveSize); }
+
+// Block barrier that orders LDS accesses only.  __syncthreads() also waits for
+// every outstanding global load of the wave; the window kernel's prologue keeps
+// loads in flight across its barriers (nothing there is handed from wave to
+// wave through global memory).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // Position of feature `fi` of a sub-class among the input keys: from the launch
@@ -740,14 +801,8 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   if (q0 >= nb_all) return;
   const int nb = min(sc.window, nb_all - q0);
 
-  // From lengths: the loads for the total in front of the window go out first,
-  // so that they share one memory latency with the loads of the window itself.
   const int fi_lo = q0 / a.B;
   using Sum = typename SumOf<IdxT>::type;
-  Sum front_part = 0;
-  if (FROM_LENGTHS)
-    front_part = prefix_partial<IdxT>(reinterpret_cast<const IdxT*>(a.offsets),
-                                      (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B), blk);
 
   // Bag q0 + i of the window: where it sits in the offsets (or lengths) array.
   auto bag_of = [&](int i, int& fi, int& b) -> int64_t {
@@ -772,8 +827,17 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     const int nfeat = min((q0 + nb - 1) / a.B - fi_lo + 1, kMaxWinFeat);
     if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = a.descs[a.feats[sc.first + fi_lo + threadIdx.x]];
   }
+  // From lengths: the total of everything in front of the window.  Its loads
+  // go out after the window's own (loads return in order: whatever is waited
+  // for first has to be issued first) and stay in flight until the scan
+  // below needs the sum.
+  PrefixSum<IdxT> front_sum;
+  if (FROM_LENGTHS)
+    front_sum.start(reinterpret_cast<const IdxT*>(a.offsets),
+                    (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B), blk);
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
-  __syncthreads();
+  lds_barrier();
+  TRA_STAMP(6);
   for (int i = threadIdx.x; i < nb; i += kCuThreads) {
     int fi, b;
     const int64_t bag = bag_of(i, fi, b);
@@ -791,7 +855,8 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
     s_slot[i] = (uint16_t)atomicAdd(&s_hist[length_bin(len)], 1);
   }
-  __syncthreads();
+  lds_barrier();
+  TRA_STAMP(7);
   if (FROM_LENGTHS) {
     __shared__ Sum s_red[kCuWaves];
     __shared__ Sum s_wave_tot[kCuWaves];
@@ -801,23 +866,26 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     // Exclusive scan of the window's lengths (window order): two bags per
     // thread, wave scan, then the 16 wave totals.  The same barrier carries
     // the block-wide total of everything in front of the window.
-    const Sum x0 = 2 * t < nb ? s_len[2 * t] : 0;
-    const Sum x1 = 2 * t + 1 < nb ? s_len[2 * t + 1] : 0;
-    Sum inc = x0 + x1;
-#pragma unroll
-    for (int off = 1; off < kWaveSize; off <<= 1) {
-      const Sum o = __shfl_up(inc, off, kWaveSize);
-      if (ln >= off) inc += o;
+    // (Only the waves that hold bags scan; every instruction that all 16 waves
+    // of the block execute costs 16 issue cycles per SIMD.)
+    const bool holds_bags = 2 * wv * kWaveSize < nb;
+    Sum x0 = 0, x1 = 0, inc = 0;
+    if (holds_bags) {
+      x0 = 2 * t < nb ? s_len[2 * t] : 0;
+      x1 = 2 * t + 1 < nb ? s_len[2 * t + 1] : 0;
+      inc = wave_scan_incl((Sum)(x0 + x1));
     }
-    const Sum front_w = wave_total_t<Sum>(front_part);
+    const Sum front_w = wave_last(wave_scan_incl(front_sum.finish()));
     if (ln == kWaveSize - 1) s_wave_tot[wv] = inc;
     if (ln == 0) s_red[wv] = front_w;
-    __syncthreads();
+    lds_barrier();
     Sum before = 0, front = 0;
 #pragma unroll
-    for (int w = 0; w < kCuWaves; ++w) {
-      if (w < wv) before += s_wave_tot[w];
-      front += s_red[w];
+    for (int w = 0; w < kCuWaves; ++w) front += s_red[w];
+    if (holds_bags) {
+#pragma unroll
+      for (int w = 0; w < kCuWaves; ++w)
+        if (w < wv) before += s_wave_tot[w];
     }
     const Sum excl = before + inc - (x0 + x1);
     // The window covers bags of features fi_lo .. fi_hi of the sub-class.  A
@@ -829,14 +897,14 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     if (one_run) {
       if (2 * t < nb) s_start[2 * t] = (int64_t)(front + excl);
       if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(front + excl + x0);
-      __syncthreads();
+      lds_barrier();
     } else {
       // General case: keep the bare scan, then add to each run what lies in
       // front of it (summed again for every run that does not continue the
       // previous one).
       if (2 * t < nb) s_start[2 * t] = (int64_t)excl;
       if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(excl + x0);
-      __syncthreads();
+      lds_barrier();
       int64_t adj = (int64_t)front;  // start = adj + scan value, for the current run
       int64_t next_pos = -1;
       for (int fi = fi_lo; fi <= fi_hi; ++fi) {
@@ -844,19 +912,20 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
         const int last = min(nb, (fi + 1) * a.B - q0);  // one past its last bag
         const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * a.B + (q0 + first - fi * a.B);
         if (fi != fi_lo && pos != next_pos) {
-          const Sum w_ = wave_total_t<Sum>(
-              prefix_partial<IdxT>(reinterpret_cast<const IdxT*>(a.offsets), pos, blk));
+          PrefixSum<IdxT> again;
+          again.start(reinterpret_cast<const IdxT*>(a.offsets), pos, blk);
+          const Sum w_ = wave_last(wave_scan_incl(again.finish()));
           if (ln == 0) s_red[wv] = w_;
-          __syncthreads();
+          lds_barrier();
           Sum total = 0;
 #pragma unroll
           for (int w = 0; w < kCuWaves; ++w) total += s_red[w];
           adj = (int64_t)total - s_start[first];
         }
         next_pos = pos + (last - first);
-        __syncthreads();  // s_red and s_start[first] have been read by everyone
+        lds_barrier();  // s_red and s_start[first] have been read by everyone
         for (int i = first + t; i < last; i += kCuThreads) s_start[i] += adj;
-        __syncthreads();
+        lds_barrier();
       }
     }
   }
@@ -873,12 +942,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
       h[k] = s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)];
       sum += h[k];
     }
-    int incl = sum;
-#pragma unroll
-    for (int d = 1; d < kWaveSize; d <<= 1) {
-      const int up = __shfl_up(incl, d, kWaveSize);
-      if (l >= d) incl += up;
-    }
+    const int incl = wave_scan_incl((int32_t)sum);
     int base = incl - sum;
 #pragma unroll
     for (int k = 0; k < kLenBins / kWaveSize; ++k) {
@@ -886,10 +950,10 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
       base += h[k];
     }
   }
-  __syncthreads();
+  lds_barrier();
   for (int i = threadIdx.x; i < nb; i += kCuThreads)
     s_order[s_hist[length_bin(s_len[i])] + s_slot[i]] = (uint16_t)i;
-  __syncthreads();
+  lds_barrier();
   TRA_STAMP(2);
 
   const int lane = threadIdx.x & (kWaveSize - 1);
