@@ -512,13 +512,19 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
 // lpr rows instead of one per row.  Needs lpr >= 2*U (a power of two): the
 // block after the current one, requested when the current one is entered, is
 // then at least two batches ahead, like the ids of pool_bag.
-template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, int NE>
+// TWO_BATCHES: lpr == 2 * U, i.e. an id block feeds exactly the two batches of
+// one loop iteration.  The block then changes at a fixed place in the loop and
+// its load is unconditional, so the number of loads in flight is the same on
+// every path and the compiler can wait for the oldest batch alone.  (Behind a
+// conditional load it has to assume the worst and drains all loads, which
+// undoes the double buffering once per iteration.)
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, int NE, bool TWO_BATCHES = false>
 __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs& a,
                                               const RowWalk& w, int64_t start64, int len,
                                               int max_len_any_lane, int lpr, int c,
                                               int group_lane0) {
   const int max_len = __builtin_amdgcn_readfirstlane(max_len_any_lane);
-  const int lpr_u = __builtin_amdgcn_readfirstlane(lpr);
+  const int lpr_u = TWO_BATCHES ? 2 * U : __builtin_amdgcn_readfirstlane(lpr);
   const IdxT start = (IdxT)start64;
   const IdxT last = (IdxT)(a.num_indices - 1);
   auto load_block = [&](int j) -> IdxT {
@@ -546,13 +552,19 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
       cur_j = j;
     }
   };
+  // The same step where it is known to happen (TWO_BATCHES: at every second batch).
+  auto advance = [&]() {
+    cur = nxt;
+    ++cur_j;
+    nxt = load_block(cur_j + 1);
+  };
   RowBuf<CB> bufA[U], bufB[U];
   int bad = 0;
 #pragma unroll
   for (int u = 0; u < U; ++u)
     bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(u), start + u, last, a, w);
   for (int it = 0; it < max_len; it += 2 * U) {
-    enter(it + U);
+    if constexpr (!TWO_BATCHES) enter(it + U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
@@ -560,7 +572,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     for (int u = 0; u < U; ++u)
       if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u]);
     if (it + U >= max_len) break;
-    enter(it + 2 * U);
+    if constexpr (TWO_BATCHES) advance(); else enter(it + 2 * U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
@@ -995,7 +1007,10 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
 #pragma unroll
     for (int k = 0; k < NE; ++k) acc[k] = 0.0f;
     if (U == 4 && lpr >= 2 * U && (lpr & (lpr - 1)) == 0)
-      pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len, lpr, c, lane - c);
+      if (lpr == 2 * U)
+        pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE, true>(acc, a, w, start, len, max_len, lpr, c, lane - c);
+      else
+        pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len, lpr, c, lane - c);
     else
       pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
     TRA_STAMP(3);
