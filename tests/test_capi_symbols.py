@@ -41,3 +41,30 @@ def test_argument_errors_are_codes_not_crashes():
     assert l.tra_cumsum(None, -1, 0, None, None, None) == -1
     assert l.tra_quantize_rows_sbhalf(None, 1, 8, 3, None, None) == -1
     assert l.tra_cumsum_workspace_bytes(10) == 0 and l.tra_cumsum_workspace_bytes(10**6) > 0
+
+
+def test_more_argument_errors():
+    """Entry points added after the first set: null and inconsistent arguments
+    come back as codes with a message, before anything touches a device."""
+    l = _lib.lib()
+    i32, i64 = ctypes.c_int32, ctypes.c_int64
+    # lengths entry
+    assert l.tra_tbe_forward_lengths(None, None, None, None, 0, None, 1, 1, 0, 0, 0, None, 0, None, None) == -1
+    assert b"null plan" in l.tra_last_error()
+    ws = l.tra_tbe_forward_lengths_workspace_bytes
+    assert ws(-1, 4, 0) == 0 and ws(26, 2048, 0) >= (26 * 2048 + 1) * 4 and ws(26, 2048, 1) > ws(26, 2048, 0)
+    # position-weighted entry: the weight description is checked first
+    one = (i32 * 1)(0)
+    assert l.tra_tbe_forward_position_weighted(None, None, None, None, 0, 0, None, 0, one, one, 1, 1, 0, 0, 0,
+                                               None, 0, None, None) == -1
+    assert b"position weight" in l.tra_last_error()
+    # per-key remap
+    assert l.tra_mch_remap_keys(None, -1, None, 0, 1, 1, None, None, None, None, None, None) == -1
+    assert l.tra_mch_remap_keys(None, 0, None, 0, 1, 1, None, None, None, None, None, None) == 0  # nothing to do
+    assert l.tra_mch_remap_keys(None, 5, None, 0, 1, 1, None, None, None, None, None, None) == -1
+    # copy: sizes and pointers in 16-byte units
+    assert l.tra_copy_bytes(None, None, 24, None) == -1 and l.tra_copy_bytes(None, None, 0, None) == 0
+    # launch description needs a plan and a buffer
+    assert l.tra_tbe_launch_info(None, 1, 1, 0, 0, None, 0) == -1
+    n = i64(0)
+    assert l.tra_tbe_error_count(None, None, ctypes.byref(n)) == -1
