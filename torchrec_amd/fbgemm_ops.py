@@ -13,7 +13,7 @@ operator that another library (fbgemm_gpu) has already defined.
 """
 from __future__ import annotations
 
-from typing import Callable, List, Optional, Tuple
+from typing import List, Optional
 
 import torch
 
