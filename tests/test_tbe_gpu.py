@@ -202,6 +202,47 @@ def test_properties_large():
     assert torch.equal(p.view(B, T, dim), a.view(B, T, dim)[:, order, :])
 
 
+def test_sequence_properties_at_scale():
+    """Sequence lookup at the shape of the unpooled workload (16 features, int8
+    x 128, 1024 samples of 0..256 ids, ~2.1 M ids; tables shortened to 100 K
+    rows), without an oracle run: a row of the output is the SUM-pooled bag that
+    holds just that id (same arithmetic, other kernel); equal ids give equal
+    rows; permuting a feature's ids permutes its rows; id -1 gives a zero row."""
+    rng = np.random.default_rng(404)
+    T, rows, dim, B = 16, 100_000, 128, 1024
+    datas = [make_table(rng, O.INT8, rows, dim) for _ in range(T)]
+    wl = [(torch.from_numpy(np.ascontiguousarray(d[:, :-4])).to(DEV), torch.from_numpy(np.ascontiguousarray(d[:, -4:])).to(DEV)) for d in datas]
+    seq = TBE(embedding_specs=[(f"t{i}", rows, dim, SparseType.INT8, EmbeddingLocation.DEVICE) for i in range(T)],
+              pooling_mode=PoolingMode.NONE, device=DEV, weight_lists=wl, output_dtype=SparseType.FP16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 256)
+    ids[rng.integers(0, len(ids), 1000)] = -1
+    ti, to = torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV)
+    out = seq(ti, to)
+    assert out.shape == (len(ids), dim) and out.dtype == torch.float16
+    # feature 3 alone through the pooled kernels, one id per bag
+    f = 3
+    lo, hi = int(offsets[f * B]), int(offsets[(f + 1) * B])
+    pooled = TBE(embedding_specs=[("t", rows, dim, SparseType.INT8, EmbeddingLocation.DEVICE)],
+                 pooling_mode=PoolingMode.SUM, device=DEV, weight_lists=[wl[f]], output_dtype=SparseType.FP16)
+    one_each = torch.arange(hi - lo + 1, dtype=ti.dtype, device=DEV)
+    want = pooled(ti[lo:hi].contiguous(), one_each)
+    assert torch.equal(out[lo:hi].view(torch.int16), want.view(torch.int16))
+    # equal ids, equal rows; -1 is a zero row
+    seg = ti[lo:hi]
+    order = torch.argsort(seg, stable=True)
+    same = seg[order][1:] == seg[order][:-1]
+    rows_sorted = out[lo:hi][order]
+    assert torch.equal(rows_sorted[1:][same], rows_sorted[:-1][same])
+    assert not out[ti == -1].any()
+    # a permutation of one feature's ids permutes its rows and leaves the others alone
+    perm = torch.randperm(hi - lo, device=DEV)
+    ti2 = ti.clone()
+    ti2[lo:hi] = seg[perm]
+    out2 = seq(ti2, to)
+    assert torch.equal(out2[lo:hi], out[lo:hi][perm])
+    assert torch.equal(out2[:lo], out[:lo]) and torch.equal(out2[hi:], out[hi:])
+
+
 # The pooled lookup has two kernels: a static bag->wave mapping for small calls
 # and a per-CU window kernel that ranks bags by length (taken when a call has
 # at least 10240 bags and 163840 ids).  TRA_BALANCED / TRA_WINDOW are the
