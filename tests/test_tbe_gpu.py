@@ -357,6 +357,41 @@ def test_window_kernel_equals_static_at_scale(monkeypatch):
     assert bits_equal(np.ascontiguousarray(a[:Bs].cpu().numpy()), want) == 0
 
 
+def test_mixed_types_weighted_at_scale(monkeypatch):
+    """The mixed workload's shape (weight types and dims mixed, weighted SUM,
+    fp32 out, 4096 samples, Poisson(30) bag lengths; 16 tables of 50 K rows):
+    several launch classes and sub-classes of the window kernel.  Same bits as
+    the static kernel; doubling every weight doubles every output exactly; a
+    sample of bags matches the oracle."""
+    rng = np.random.default_rng(303)
+    dts = [O.INT8, O.INT4, O.INT2, O.FP16]
+    dims = [32, 64, 128, 256]
+    T, rows, B = 16, 50_000, 4096
+    specs = [(dts[t % 4], rows, dims[(t // 4) % 4]) for t in range(T)]
+    ftm = list(range(T))
+    tbe, store = build(rng, specs, ftm, O.SUM, O.FP32, 16)
+    lengths = rng.poisson(30, T * B).astype(np.int32)
+    offsets = np.zeros(T * B + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(lengths)
+    ids = rng.integers(0, rows, int(offsets[-1])).astype(np.int32)
+    psw = rng.uniform(0, 1, len(ids)).astype(np.float32)
+    ti, to, tw = (torch.from_numpy(x).to(DEV) for x in (ids, offsets, psw))
+    monkeypatch.delenv("TRA_BALANCED", raising=False)
+    a = tbe(ti, to, tw)
+    monkeypatch.setenv("TRA_BALANCED", "0")
+    b = tbe(ti, to, tw)
+    monkeypatch.delenv("TRA_BALANCED")
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    assert torch.equal(tbe(ti, to, tw * 2), a * 2)
+    Bs = 8
+    sub_len = lengths.reshape(T, B)[:, :Bs]
+    sub_off = np.zeros(T * Bs + 1, dtype=np.int32)
+    sub_off[1:] = np.cumsum(sub_len.reshape(-1))
+    pick = np.concatenate([np.arange(offsets[f * B], offsets[f * B + Bs]) for f in range(T)])
+    want = O.tbe_forward(store, ftm, Bs, ids[pick], sub_off, psw[pick], O.SUM, O.FP32)
+    assert bits_equal(np.ascontiguousarray(a[:Bs].cpu().numpy()), want) == 0
+
+
 def test_lookup_under_hip_graph():
     """The lookup captured in a HIP graph: several replays, with eager work and
     synchronisation in between, each equal to the eager result."""
