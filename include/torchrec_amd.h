@@ -288,6 +288,19 @@ int tra_mch_remap_keys(const void* values, int64_t n, const void* offsets, int32
                        const int64_t* miss_id, void* out, void* stream);
 
 /* Measurement ------------------------------------------------------------- */
+/* Column regroup of pooled outputs ------------------------------------------- */
+/* Copies num_blocks column blocks between row-major matrices of `rows` rows:
+ * block k is width[k] elements of every row, read at src[k] with row stride
+ * src_stride[k] and written at dst[k] with row stride dst_stride[k] (strides in
+ * elements; both pointers include the block's first column; elements of 2 or 4
+ * bytes).  src, dst and the three arrays are HOST arrays.  One launch per 96
+ * blocks.  Replaces the column gather behind KeyedTensor.regroup
+ * (torch.ops.fbgemm.permute_pooled_embs / permute_multi_embedding or one
+ * torch.cat, torchrec/sparse/jagged_tensor.py:146-172, 191-239, 3326-3344). */
+int tra_regroup_columns(const void* const* src, const int64_t* src_stride, void* const* dst,
+                        const int64_t* dst_stride, const int32_t* width, int32_t num_blocks,
+                        int64_t rows, int32_t elem_bytes, void* stream);
+
 /* Streaming device-to-device copy of `bytes` bytes (a multiple of 16, 16-byte
  * aligned pointers) by a kernel named tra_copy_kernel.  A copy of known size
  * under the same hardware counters calibrates FETCH_SIZE / WRITE_SIZE readings

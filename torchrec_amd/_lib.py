@@ -42,6 +42,7 @@ EXPORTED_SYMBOLS = [
     "tra_position_weights",
     "tra_mch_remap",
     "tra_mch_remap_keys",
+    "tra_regroup_columns",
     "tra_copy_bytes",
 ]
 
@@ -110,6 +111,10 @@ def lib() -> ctypes.CDLL:
         l.tra_mch_remap_keys.argtypes = [
             vp, i64, vp, i32, i32, i32, ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(i64),
             ctypes.POINTER(i64), vp, vp,
+        ]
+        l.tra_regroup_columns.argtypes = [
+            ctypes.POINTER(vp), ctypes.POINTER(i64), ctypes.POINTER(vp), ctypes.POINTER(i64), ctypes.POINTER(i32),
+            i32, i64, i32, vp,
         ]
         l.tra_copy_bytes.argtypes = [vp, vp, i64, vp]
         _lib = l

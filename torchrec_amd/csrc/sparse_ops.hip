@@ -402,6 +402,36 @@ __global__ void mch_remap_keys_kernel(const void* values, int64_t n, const void*
   }
 }
 
+// Column blocks of row-major matrices copied into other matrices: block k is
+// `width` elements of every row, from src[k] (row stride src_stride[k]) to
+// dst[k] (row stride dst_stride[k]); both pointers already include the
+// block's first column.  blockIdx.y is the block, blockIdx.x strides over its
+// rows * width elements.  E = element size in bytes (2 or 4).
+constexpr int kRegroupBlocks = 96;
+struct RegroupBlocks {
+  const void* src[kRegroupBlocks];
+  void* dst[kRegroupBlocks];
+  int64_t src_stride[kRegroupBlocks];
+  int64_t dst_stride[kRegroupBlocks];
+  int32_t width[kRegroupBlocks];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void regroup_kernel(const RegroupBlocks b, int64_t rows) {
+  const int k = blockIdx.y;
+  const T* __restrict__ src = reinterpret_cast<const T*>(b.src[k]);
+  T* __restrict__ dst = reinterpret_cast<T*>(b.dst[k]);
+  const int64_t ss = b.src_stride[k], ds = b.dst_stride[k];
+  const int w = b.width[k];
+  const int64_t n = rows * w;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int64_t r = i / w;
+    const int c = (int)(i - r * w);
+    dst[r * ds + c] = src[r * ss + c];
+  }
+}
+
 // Plain streaming copy, 16 bytes per lane per step.
 __global__ __launch_bounds__(256) void tra_copy_kernel(const uint4* __restrict__ src,
                                                         uint4* __restrict__ dst, int64_t n16) {
@@ -756,6 +786,53 @@ int tra_mch_remap_keys(const void* values, int64_t n, const void* offsets, int32
       hipLaunchKernelGGL(mch_remap_keys_kernel<int32_t>, dim3(gx, nk), dim3(256), 0, (hipStream_t)stream,
                          values, n, offsets, batch_size, t, out);
     const int rc = check_launch("tra_mch_remap_keys");
+    if (rc != TRA_OK) return rc;
+  }
+  return TRA_OK;
+}
+
+int tra_regroup_columns(const void* const* src, const int64_t* src_stride, void* const* dst,
+                        const int64_t* dst_stride, const int32_t* width, int32_t num_blocks,
+                        int64_t rows, int32_t elem_bytes, void* stream) {
+  if (num_blocks < 0 || rows < 0) {
+    set_error("tra_regroup_columns: negative size");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (elem_bytes != 2 && elem_bytes != 4) {
+    set_error("tra_regroup_columns: element size %d (2 or 4 bytes are supported)", elem_bytes);
+    return TRA_ERR_UNSUPPORTED;
+  }
+  if (num_blocks == 0 || rows == 0) return TRA_OK;
+  if (!src || !dst || !src_stride || !dst_stride || !width) {
+    set_error("tra_regroup_columns: null argument");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  int64_t widest = 0;
+  for (int k = 0; k < num_blocks; ++k) {
+    if (!src[k] || !dst[k] || width[k] < 0 || src_stride[k] < width[k] || dst_stride[k] < width[k]) {
+      set_error("tra_regroup_columns: block %d is null or wider than its row stride", k);
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+    widest = std::max<int64_t>(widest, width[k]);
+  }
+  if (widest == 0) return TRA_OK;
+  const unsigned gx = (unsigned)std::max<int64_t>(1, std::min<int64_t>((rows * widest + 255) / 256, 2048));
+  for (int k0 = 0; k0 < num_blocks; k0 += kRegroupBlocks) {
+    const int nk = std::min(kRegroupBlocks, num_blocks - k0);
+    RegroupBlocks b;
+    std::memset(&b, 0, sizeof(b));
+    for (int k = 0; k < nk; ++k) {
+      b.src[k] = src[k0 + k];
+      b.dst[k] = dst[k0 + k];
+      b.src_stride[k] = src_stride[k0 + k];
+      b.dst_stride[k] = dst_stride[k0 + k];
+      b.width[k] = width[k0 + k];
+    }
+    if (elem_bytes == 2)
+      hipLaunchKernelGGL(regroup_kernel<uint16_t>, dim3(gx, nk), dim3(256), 0, (hipStream_t)stream, b, rows);
+    else
+      hipLaunchKernelGGL(regroup_kernel<uint32_t>, dim3(gx, nk), dim3(256), 0, (hipStream_t)stream, b, rows);
+    const int rc = check_launch("tra_regroup_columns");
     if (rc != TRA_OK) return rc;
   }
   return TRA_OK;

@@ -644,6 +644,82 @@ class KeyedJaggedTensor:
         return "KeyedJaggedTensor({\n" + ",\n".join(parts) + "\n})\n"
 
 
+def _regroup_plan(keyed_tensors: List[KeyedTensor], groups: List[List[str]]):
+    """Per group the (keyed tensor index, first column, width) of every block, in order."""
+    where: Dict[str, Tuple[int, int, int]] = {}
+    for t, kt in enumerate(keyed_tensors):
+        offsets = kt.offset_per_key()
+        for i, key in enumerate(kt.keys()):
+            where[key] = (t, offsets[i], kt.length_per_key()[i])
+    return [[where[name] for name in group] for group in groups]
+
+
+def _regroup_keyed_tensors(keyed_tensors: List[KeyedTensor], groups: List[List[str]]) -> List[torch.Tensor]:
+    """Regroup with plain slicing and concatenation (jagged_tensor.py:146-172): the
+    form used for host tensors and the yardstick for the kernel."""
+    key_dim = keyed_tensors[0].key_dim()
+    out = []
+    for blocks in _regroup_plan(keyed_tensors, groups):
+        parts = [keyed_tensors[t].values().narrow(key_dim, col, width) for t, col, width in blocks]
+        if not parts:  # an empty group: no columns
+            parts = [keyed_tensors[0].values().narrow(key_dim, 0, 0)]
+        out.append(torch.cat(parts, dim=key_dim))
+    return out
+
+
+def regroup_kts(keyed_tensors: List[KeyedTensor], groups: List[List[str]]) -> List[torch.Tensor]:
+    """KeyedTensor.regroup (jagged_tensor.py:209-239).  Two-dimensional fp16 / bf16 /
+    fp32 tensors on the GPU (the pooled lookup's outputs) are regrouped by one
+    launch of the column-copy kernel for all groups; anything else by slicing."""
+    first = keyed_tensors[0].values()
+    on_gpu = (
+        first.device.type == "cuda"
+        and keyed_tensors[0].key_dim() == 1
+        and all(
+            kt.values().dim() == 2 and kt.key_dim() == 1 and kt.values().dtype == first.dtype
+            and kt.values().device == first.device and kt.values().stride(1) == 1
+            and kt.values().shape[0] == first.shape[0]
+            for kt in keyed_tensors
+        )
+        and first.element_size() in (2, 4)
+    )
+    if not on_gpu:
+        return _regroup_keyed_tensors(keyed_tensors, groups)
+    import ctypes
+
+    from torchrec_amd import _lib
+
+    plan = _regroup_plan(keyed_tensors, groups)
+    rows, esz = first.shape[0], first.element_size()
+    outs = [torch.empty((rows, sum(w for _, _, w in blocks)), dtype=first.dtype, device=first.device) for blocks in plan]
+    src, src_stride, dst, dst_stride, width = [], [], [], [], []
+    for blocks, out in zip(plan, outs):
+        col_out = 0
+        for t, col, w in blocks:
+            v = keyed_tensors[t].values()
+            src.append(v.data_ptr() + col * esz)
+            src_stride.append(v.stride(0))
+            dst.append(out.data_ptr() + col_out * esz)
+            dst_stride.append(out.stride(0) if out.shape[1] else 1)
+            width.append(w)
+            col_out += w
+    n = len(src)
+    if n and rows:
+        vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
+        _lib.check(
+            _lib.lib().tra_regroup_columns(
+                (vp * n)(*src), (i64 * n)(*src_stride), (vp * n)(*dst), (i64 * n)(*dst_stride), (i32 * n)(*width),
+                n, rows, esz, _lib.current_stream(first.device),
+            )
+        )
+    return outs
+
+
+def permute_multi_embedding(keyed_tensors: List[KeyedTensor], groups: List[List[str]]) -> List[torch.Tensor]:
+    """Same result as ``regroup_kts`` (jagged_tensor.py:191-206)."""
+    return regroup_kts(keyed_tensors, groups)
+
+
 class ComputeKJTToJTDict(torch.nn.Module):
     """Module form of KeyedJaggedTensor.to_dict (jagged_tensor.py:1320-1361)."""
 
@@ -753,6 +829,21 @@ class KeyedTensor:
     def to_dict(self) -> Dict[str, torch.Tensor]:
         pieces = torch.split(self._values, self._length_per_key, dim=self._key_dim)
         return {key: pieces[i] for i, key in enumerate(self._keys)}
+
+    @staticmethod
+    def regroup(keyed_tensors: List["KeyedTensor"], groups: List[List[str]]) -> List[torch.Tensor]:
+        """One tensor per group: the named blocks of the given KeyedTensors
+        concatenated along ``key_dim`` in the group's order (a key may be used
+        several times or not at all; of a key that several KeyedTensors hold,
+        the last one's block is taken).  jagged_tensor.py:3326-3344."""
+        return regroup_kts(keyed_tensors, groups)
+
+    @staticmethod
+    def regroup_as_dict(
+        keyed_tensors: List["KeyedTensor"], groups: List[List[str]], keys: List[str]
+    ) -> Dict[str, torch.Tensor]:
+        assert len(groups) == len(keys), "Groups and keys should have same length"
+        return dict(zip(keys, KeyedTensor.regroup(keyed_tensors, groups)))
 
     def to(self, device: torch.device, non_blocking: bool = False) -> "KeyedTensor":
         return KeyedTensor(
