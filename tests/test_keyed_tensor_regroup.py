@@ -77,3 +77,34 @@ def test_regroup_kernel_against_slicing(dtype):
     part = KeyedTensor(keys=["x", "y"], length_per_key=[30, 20], values=wide[:, 10:60])
     got = regroup_kts([part], [["y", "x"]])
     assert torch.equal(got[0], torch.cat([wide[:, 40:60], wide[:, 10:40]], 1))
+
+
+@pytest.mark.parametrize("dev", DEVICES)
+def test_kt_regroup_as_dict_module(dev):
+    """torchrec/modules/tests/test_regroup.py: same result as the static method,
+    on the first and on later batches; a duplicate key is refused; the cast."""
+    from torchrec_amd.modules.embedding_configs import DataType
+    from torchrec_amd.modules.regroup import KTRegroupAsDict
+
+    def batch():
+        t1 = [torch.randn(6, 4, device=dev), torch.randn(6, 8, device=dev), torch.randn(6, 2, device=dev)]
+        t2 = [torch.randn(6, 3, device=dev), torch.randn(6, 10, device=dev)]
+        return [KeyedTensor.from_tensor_list(["f1", "f2", "f3"], t1), KeyedTensor.from_tensor_list(["g1", "g2"], t2)]
+
+    groups, keys = [["f1", "g2", "f3"], ["f2", "g1"]], ["object", "user"]
+    m = KTRegroupAsDict(groups, keys)
+    for _ in range(3):
+        kts = batch()
+        got, want = m(kts), KeyedTensor.regroup_as_dict(kts, groups, keys)
+        assert list(got) == keys and all(torch.equal(got[k], want[k]) for k in keys)
+    half = KTRegroupAsDict(groups, keys, emb_dtype=DataType.FP16)
+    kts = batch()
+    out = half(kts)
+    assert out["user"].dtype == torch.float16
+    assert torch.equal(out["user"], torch.cat([kts[0]["f2"], kts[1]["g1"]], 1).half())
+    dup = [KeyedTensor.from_tensor_list(["f1"], [torch.randn(2, 2, device=dev)]),
+           KeyedTensor.from_tensor_list(["f1"], [torch.randn(2, 2, device=dev)])]
+    with pytest.raises(RuntimeError, match="Duplicate key"):
+        KTRegroupAsDict([["f1"]], ["a"])(dup)
+    m.clear_cache()
+    assert not m._is_inited

@@ -667,10 +667,12 @@ def _regroup_keyed_tensors(keyed_tensors: List[KeyedTensor], groups: List[List[s
     return out
 
 
-def regroup_kts(keyed_tensors: List[KeyedTensor], groups: List[List[str]]) -> List[torch.Tensor]:
+def regroup_kts(keyed_tensors: List[KeyedTensor], groups: List[List[str]], plan=None) -> List[torch.Tensor]:
     """KeyedTensor.regroup (jagged_tensor.py:209-239).  Two-dimensional fp16 / bf16 /
     fp32 tensors on the GPU (the pooled lookup's outputs) are regrouped by one
-    launch of the column-copy kernel for all groups; anything else by slicing."""
+    launch of the column-copy kernel for all groups; anything else by slicing.
+    ``plan`` is a ``_regroup_plan`` result kept by a caller whose key layout does
+    not change."""
     first = keyed_tensors[0].values()
     on_gpu = (
         first.device.type == "cuda"
@@ -689,7 +691,8 @@ def regroup_kts(keyed_tensors: List[KeyedTensor], groups: List[List[str]]) -> Li
 
     from torchrec_amd import _lib
 
-    plan = _regroup_plan(keyed_tensors, groups)
+    if plan is None:
+        plan = _regroup_plan(keyed_tensors, groups)
     rows, esz = first.shape[0], first.element_size()
     outs = [torch.empty((rows, sum(w for _, _, w in blocks)), dtype=first.dtype, device=first.device) for blocks in plan]
     src, src_stride, dst, dst_stride, width = [], [], [], [], []
