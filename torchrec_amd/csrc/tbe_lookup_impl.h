@@ -675,7 +675,7 @@ struct SumOf<int32_t> { using type = int32_t; };
 // This thread's share of sum(lengths[0 .. p)).  The block reads the range 16
 // bytes per lane per step, kPrefixBatch independent loads at a time (a lane's
 // index past the end is clamped and its value dropped, so no load is
-// predicated per lane; steps past the end are skipped for the whole wave).
+// predicated).
 // start() adds up every batch but the last and leaves the last one in flight;
 // finish() adds it, so the last round trip overlaps whatever the caller does
 // between the two calls.
@@ -701,20 +701,24 @@ struct PrefixSum {
     const int j = k + rot;
     return (j >= nk ? j - nk : j) * kCuThreads + (int)threadIdx.x;
   }
+  // Always kPrefixBatch loads: were their number to depend on the data, the
+  // compiler could not wait for an older load without draining these.  A step
+  // past the end reads element 0 in every lane (a single request).
   __device__ __forceinline__ void issue(int k0) {
 #pragma unroll
-    for (int k = 0; k < kPrefixBatch; ++k)
-      if (k0 + k < nk) x[k] = vin[min(index_of(k0 + k), nvec - 1)];
+    for (int k = 0; k < kPrefixBatch; ++k) {
+      const int idx = k0 + k < nk ? min(index_of(k0 + k), nvec - 1) : 0;
+      x[k] = vin[idx];
+    }
   }
   __device__ __forceinline__ void consume(int k0) {
 #pragma unroll
-    for (int k = 0; k < kPrefixBatch; ++k)
-      if (k0 + k < nk) {
-        S sum = 0;
+    for (int k = 0; k < kPrefixBatch; ++k) {
+      S sum = 0;
 #pragma unroll
-        for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
-        part += index_of(k0 + k) < nvec ? sum : (S)0;
-      }
+      for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
+      part += (k0 + k < nk && index_of(k0 + k) < nvec) ? sum : (S)0;
+    }
   }
   __device__ __forceinline__ void start(const IdxT* __restrict__ lengths, int64_t p, int rot_) {
     vin = reinterpret_cast<const Vec*>(lengths);
