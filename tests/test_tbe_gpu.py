@@ -392,6 +392,44 @@ def test_mixed_types_weighted_at_scale(monkeypatch):
     assert bits_equal(np.ascontiguousarray(a[:Bs].cpu().numpy()), want) == 0
 
 
+@pytest.mark.parametrize("from_lengths", [False, True])
+def test_window_kernel_many_features(monkeypatch, from_lengths):
+    """More features than the window kernel keeps close at hand: 300 features
+    on three tables (over 128 per launch class: key positions then come from
+    the descriptors, not the launch arguments), 3 samples each, 128 bags per
+    window (over 32 features per window: their descriptors are read from global
+    memory, not from LDS), keys in reverse order."""
+    monkeypatch.setenv("TRA_BALANCED", "1")
+    monkeypatch.setenv("TRA_WINDOW", "128")
+    rng = np.random.default_rng(300)
+    F, B = 300, 3
+    specs = [(O.INT4, 400, 64), (O.INT8, 300, 64), (O.INT4, 500, 32)]
+    ftm = [f % 3 for f in range(F)]
+    tbe, store = build(rng, specs, ftm, O.SUM, O.FP32, 16)
+    rows_f = [specs[t][1] for t in ftm]
+    lengths, offsets, ids = make_bags(rng, rows_f, B, 12)
+    want = O.tbe_forward(store, ftm, B, ids, offsets, None, O.SUM, O.FP32)
+    ti = torch.from_numpy(ids).to(DEV)
+    if from_lengths:
+        got = tbe(ti, None, lengths=torch.from_numpy(lengths.astype(np.int32)).to(DEV), batch_size=B)
+    else:
+        got = tbe(ti, torch.from_numpy(offsets).to(DEV))
+    assert bits_equal(got.cpu().numpy(), want) == 0
+    # the same bags addressed through a reversed key order
+    rev = list(range(F - 1, -1, -1))
+    L = lengths.reshape(F, B)
+    seg = [ids[offsets[f * B]:offsets[(f + 1) * B]] for f in range(F)]
+    r_len = np.concatenate([L[f] for f in rev]).astype(np.int32)
+    r_off = np.zeros(F * B + 1, dtype=np.int32)
+    r_off[1:] = np.cumsum(r_len)
+    r_ids = torch.from_numpy(np.concatenate([seg[f] for f in rev])).to(DEV)
+    if from_lengths:
+        got = tbe(r_ids, None, lengths=torch.from_numpy(r_len).to(DEV), batch_size=B, feature_positions=rev)
+    else:
+        got = tbe(r_ids, torch.from_numpy(r_off).to(DEV), batch_size=B, feature_positions=rev)
+    assert bits_equal(got.cpu().numpy(), want) == 0
+
+
 def test_lookup_under_hip_graph():
     """The lookup captured in a HIP graph: several replays, with eager work and
     synchronisation in between, each equal to the eager result."""
