@@ -122,7 +122,9 @@ class PositionWeightedModuleCollection(FeatureProcessorsCollection, CopyMixIn):
 
     def _table(self, keys: List[str], dev: torch.device) -> torch.Tensor:
         """The weight vectors of ``keys`` in one fp32 tensor.  Rebuilt only when a
-        parameter was replaced or written to since the last call."""
+        parameter was replaced or written to since the last call (its version
+        counter moved; a write through ``.data`` does not move it: call
+        ``_resync()`` after one)."""
         present = [self.position_weights_dict[k] for k in keys if k in self.position_weights_dict]
         stamp = (tuple(keys), dev, tuple((id(p), p._version) for p in present))
         if self._table_cache is None or self._table_cache[0] != stamp:
