@@ -102,7 +102,8 @@ int tra_tbe_destroy(tra_tbe_t tbe);
  * Arithmetic per output column, ids in order: acc = fmaf(w*scale, q, acc +
  * w*bias) (fp16/fp32 rows: acc = fmaf(w, x, acc)); MEAN multiplies by 1.0f/len;
  * output rounded to nearest even.  Ids outside [0, rows) other than -1 are
- * skipped and counted (tra_tbe_error_count). */
+ * skipped and counted (tra_tbe_error_count).  Every buffer sits at a multiple
+ * of its element size (weights: 4 bytes), else TRA_ERR_INVALID_ARGUMENT. */
 int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
                     const void* offsets, int32_t idx_is_i64,
                     const float* per_sample_weights, int32_t batch_size,

@@ -376,3 +376,61 @@ def test_position_weighted_entry_checks_its_layout():
         op(ids, offsets, position_weights=(table, [-1], [3]))
     with pytest.raises(AssertionError):
         op(ids, offsets, position_weights=(table, [], []))
+
+
+@pytest.mark.gpu
+def test_forward_rejects_misaligned_buffers():
+    """Ids, bag boundaries, weights and the output must sit at multiples of
+    their element size: the C entry point says so instead of launching."""
+    from torchrec_amd import _lib
+
+    dev = torch.device("cuda:0")
+    rows, D, B = 50, 32, 4
+    q = torch.from_numpy(O.quantize_sbhalf(np.zeros((rows, D), dtype=np.float32), 8))
+    cfg = EmbeddingBagConfig(name="t", embedding_dim=D, num_embeddings=rows, feature_names=["f"], data_type=DataType.INT8)
+    m = QuantEBC([cfg], True, dev, table_name_to_quantized_weights={"t": (q[:, :-4].to(dev), q[:, -4:].to(dev))})
+    op = m._emb_modules[0]
+    ids = torch.zeros(10, dtype=torch.int64, device=dev)
+    offsets = torch.arange(0, 10, 2, dtype=torch.int64, device=dev)
+    out = torch.empty(B, D, dtype=torch.float32, device=dev)
+    l, plan, stream = _lib.lib(), op._get_plan(None), _lib.current_stream(dev)
+
+    def call(w, i, o, dst):
+        return l.tra_tbe_forward(plan, w, i, o, 1, None, B, 8, 0, _lib.FP32, dst, D, stream)
+
+    w = op.weights_dev.data_ptr()
+    assert call(w, ids.data_ptr(), offsets.data_ptr(), out.data_ptr()) == 0
+    for args in (
+        (w + 2, ids.data_ptr(), offsets.data_ptr(), out.data_ptr()),
+        (w, ids.data_ptr() + 4, offsets.data_ptr(), out.data_ptr()),
+        (w, ids.data_ptr(), offsets.data_ptr() + 4, out.data_ptr()),
+        (w, ids.data_ptr(), offsets.data_ptr(), out.data_ptr() + 2),
+    ):
+        assert call(*args) == -1 and b"aligned" in l.tra_last_error()
+    torch.cuda.synchronize()
+
+
+@pytest.mark.gpu
+def test_operator_built_on_cpu_then_moved():
+    """An operator filled on the CPU and moved with ``.to()`` looks up like one
+    built on the GPU."""
+    from torchrec_amd.tbe import PoolingMode
+    from torchrec_amd.tbe.split_table_batched_embeddings_ops_inference import IntNBitTableBatchedEmbeddingBagsCodegen
+
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(5)
+    rows, D, B = 200, 64, 16
+    q = torch.from_numpy(O.quantize_sbhalf(rng.standard_normal((rows, D)).astype(np.float32), 4))
+    pair = [(q[:, :-4].contiguous(), q[:, -4:].contiguous())]
+    spec = [("t", rows, D, SparseType.INT4, None)]
+    on_gpu = IntNBitTableBatchedEmbeddingBagsCodegen(
+        spec, device=dev, pooling_mode=PoolingMode.SUM, weight_lists=[(w.to(dev), s.to(dev)) for w, s in pair]
+    )
+    moved = IntNBitTableBatchedEmbeddingBagsCodegen(
+        spec, device=torch.device("cpu"), pooling_mode=PoolingMode.SUM, weight_lists=pair
+    ).to(dev)
+    assert moved.current_device == dev and moved.weights_dev.is_cuda
+    lengths = torch.from_numpy(rng.integers(0, 9, size=B).astype(np.int32))
+    ids = torch.from_numpy(rng.integers(0, rows, size=int(lengths.sum())).astype(np.int32)).to(dev)
+    offsets = torch.cat([torch.zeros(1, dtype=torch.int32), lengths.cumsum(0).int()]).to(dev)
+    assert torch.equal(on_gpu(ids, offsets), moved(ids, offsets))

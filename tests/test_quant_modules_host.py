@@ -177,3 +177,19 @@ def test_create_on_meta_device_without_providing_weights():
     qec = QEC([EmbeddingConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1"])],
               device=torch.device("meta"))
     assert qec.state_dict()["embeddings.t1.weight"].device.type == "meta"
+
+
+def test_operator_follows_its_buffer_between_devices():
+    """``.to()`` moves the packed buffer; the operator's launch device follows
+    and a lookup away from the GPU still fails with a message, not a fault."""
+    from torchrec_amd.tbe.split_table_batched_embeddings_ops_inference import IntNBitTableBatchedEmbeddingBagsCodegen
+
+    op = IntNBitTableBatchedEmbeddingBagsCodegen(
+        [("t", 10, 8, SparseType.INT8, None)], device=CPU, pooling_mode=PoolingMode.SUM
+    )
+    op.initialize_weights()
+    assert op.current_device == CPU and op.weights_dev.device == CPU
+    op.to("meta")
+    assert op.current_device.type == "meta" and op.weights_dev.device.type == "meta"
+    with pytest.raises(_lib.TorchrecAmdError, match="MI355X"):
+        op(torch.zeros(2, dtype=torch.int32), torch.tensor([0, 2], dtype=torch.int32))

@@ -711,7 +711,7 @@ int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys, 
   }
   const int64_t n = (int64_t)num_keys * batch_size;
   if (n == 0) return TRA_OK;
-  if (!offsets || !key_start || !key_len) {
+  if (!offsets || !key_start || !key_len || !out) {
     set_error("tra_position_weights: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
   }

@@ -365,6 +365,17 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     set_error("tra_tbe_forward: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
   }
+  {
+    // Rows are read as dwords; ids, bag boundaries and weights as whole elements.
+    const uintptr_t isz = idx_is_i64 ? 8 : 4;
+    if ((uintptr_t)weights % 4 != 0 || (uintptr_t)indices % isz != 0 ||
+        (uintptr_t)offsets % isz != 0 || (uintptr_t)per_sample_weights % 4 != 0 ||
+        (uintptr_t)out % (out_dtype == TRA_FP16 ? 2 : 4) != 0 ||
+        (pw != nullptr && (uintptr_t)pw->table % 4 != 0)) {
+      set_error("tra_tbe_forward: a buffer is not aligned to its element size");
+      return TRA_ERR_INVALID_ARGUMENT;
+    }
+  }
   if (nobag && !tbe->same_dim) {
     set_error("tra_tbe_forward: sequence lookup needs one embedding dim for all tables");
     return TRA_ERR_INVALID_ARGUMENT;

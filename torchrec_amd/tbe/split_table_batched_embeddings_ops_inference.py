@@ -157,6 +157,19 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             self.weight_initialized = True
             self._drop_plan()
 
+    def _apply(self, fn, recurse: bool = True):  # type: ignore[no-untyped-def]
+        """``.to()`` / ``.cuda()`` / ``.cpu()`` move the packed buffer; the device the
+        operator launches on follows it, and plans made for the old device go."""
+        super()._apply(fn, recurse)
+        dev = self.weights_dev.device
+        if dev.type == "cuda" and dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
+        if dev != self.current_device:
+            self.current_device = dev
+            self._drop_plan()
+            self._workspace.clear()
+        return self
+
     def _num_keys_of(self, positions: Tuple[int, ...]) -> int:
         """Smallest number of KJT keys that covers ``positions`` (remembered per placement)."""
         n = self._num_keys.get(positions)
@@ -302,6 +315,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             )
         if not self._weights_initialized:
             raise _lib.TorchrecAmdError("weights are not initialized (call initialize_weights())")
+        if self.weights_dev.device != dev:  # e.g. the buffer was replaced by hand
+            raise _lib.TorchrecAmdError(f"packed weights are on {self.weights_dev.device}, the operator on {dev}")
         _lib.require_gpu(indices, "indices")
         if indices.dtype not in (torch.int32, torch.int64):
             raise TypeError(f"indices must be int32 or int64, got {indices.dtype}")
