@@ -548,6 +548,28 @@ def test_forward_from_lengths_at_scale():
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+@pytest.mark.parametrize("B,idt", [(8192, np.int32), (4096, np.int64)])
+def test_forward_from_lengths_long_prefix(B, idt):
+    """Enough bags that the blocks of the last windows sum the lengths in front
+    of them in many batches of loads (26 x 8192 int32 lengths, 26 x 4096 int64
+    ones): lengths entry == offsets entry, bit for bit, and the launch really
+    is the from-lengths one."""
+    rng = np.random.default_rng(77 + B)
+    T, rows, dim = 26, 20_000, 64
+    tbe, store = build(rng, [(O.INT8, rows, dim)] * T, list(range(T)), O.MEAN, O.FP32, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 12, idt, empty_frac=0.1)
+    psw = torch.from_numpy(rng.uniform(-1, 1, len(ids)).astype(np.float32)).to(DEV)
+    ti = torch.from_numpy(ids).to(DEV)
+    a = tbe(ti, torch.from_numpy(offsets).to(DEV), psw)
+    b = tbe(ti, None, psw, lengths=torch.from_numpy(lengths).to(DEV), batch_size=B)
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    import ctypes
+    from torchrec_amd import _lib
+    buf = ctypes.create_string_buffer(512)
+    _lib.check(_lib.lib().tra_tbe_launch_info(tbe._get_plan(None), B, len(ids), int(tbe.pooling_mode), T, buf, 512))
+    assert b"from_lengths" in buf.value
+
+
 def test_table_beyond_2_31_rows():
     """A table with more than 2^31 rows (fp32, dim 1: 8.6 GB): int64 ids beyond 2^31 address the
     right rows; int32 ids see every non-negative id as in range; ids >= rows are skipped and counted."""

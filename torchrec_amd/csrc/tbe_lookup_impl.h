@@ -704,21 +704,22 @@ struct PrefixSum {
   // Always kPrefixBatch loads: were their number to depend on the data, the
   // compiler could not wait for an older load without draining these.  A step
   // past the end reads element 0 in every lane (a single request).
+  __device__ __forceinline__ Vec fetch(int k) const {
+    return vin[k < nk ? min(index_of(k), nvec - 1) : 0];
+  }
+  __device__ __forceinline__ void add(int k, const Vec& v) {
+    S sum = 0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) sum += (S)v.v[i];
+    part += (k < nk && index_of(k) < nvec) ? sum : (S)0;
+  }
   __device__ __forceinline__ void issue(int k0) {
 #pragma unroll
-    for (int k = 0; k < kPrefixBatch; ++k) {
-      const int idx = k0 + k < nk ? min(index_of(k0 + k), nvec - 1) : 0;
-      x[k] = vin[idx];
-    }
+    for (int k = 0; k < kPrefixBatch; ++k) x[k] = fetch(k0 + k);
   }
   __device__ __forceinline__ void consume(int k0) {
 #pragma unroll
-    for (int k = 0; k < kPrefixBatch; ++k) {
-      S sum = 0;
-#pragma unroll
-      for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
-      part += (k0 + k < nk && index_of(k0 + k) < nvec) ? sum : (S)0;
-    }
+    for (int k = 0; k < kPrefixBatch; ++k) add(k0 + k, x[k]);
   }
   __device__ __forceinline__ void start(const IdxT* __restrict__ lengths, int64_t p, int rot_) {
     vin = reinterpret_cast<const Vec*>(lengths);
@@ -732,11 +733,17 @@ struct PrefixSum {
     tail = lengths[max(min(ti, p - 1), (int64_t)0)];
     if ((int64_t)threadIdx.x >= rest) tail = 0;
     k_last = nk > 0 ? ((nk - 1) / kPrefixBatch) * kPrefixBatch : 0;
+    // kPrefixBatch loads stay in flight: each step adds the oldest (loads
+    // return in issue order) and puts the load of the step one batch ahead
+    // in its place.  The last batch is left for finish().
+    issue(0);
     for (int k0 = 0; k0 < k_last; k0 += kPrefixBatch) {
-      issue(k0);
-      consume(k0);
+#pragma unroll
+      for (int k = 0; k < kPrefixBatch; ++k) {
+        add(k0 + k, x[k]);
+        x[k] = fetch(k0 + kPrefixBatch + k);
+      }
     }
-    issue(k_last);
   }
   __device__ __forceinline__ S finish() {
     consume(k_last);
