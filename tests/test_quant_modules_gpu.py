@@ -242,3 +242,45 @@ def test_qebc_kjt_from_lengths_equals_from_offsets():
     b = m(KeyedJaggedTensor(keys=keys, values=values, offsets=offsets))
     assert a.keys() == b.keys() and torch.equal(a.values(), b.values())
     assert torch.isfinite(a.values()).all()
+
+
+@pytest.mark.parametrize("from_lengths", [True, False])
+def test_forwards_in_flight_on_several_streams(from_lengths):
+    """Independent requests on separate HIP streams (a serving loop): lookups of
+    one module overlap on the GPU and every one gives the bits it gives alone.
+    Large enough for the per-CU window kernel, whose blocks of consecutive
+    launches then share the chip."""
+    dev = DEV
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    T, B, rows = 8, 2048, 20_000
+    tables = [EmbeddingBagConfig(name=f"t{t}", embedding_dim=64, num_embeddings=rows, feature_names=[f"f{t}"],
+                                 data_type=DataType.INT4, pooling=PoolingType.SUM) for t in range(T)]
+    m = QuantEBC(tables, True, dev, output_dtype=torch.half)
+    for tbe in m._emb_modules:
+        tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, generator=gen).to(dev))
+        for t in range(len(tbe.rows)):  # finite fp16 scale/bias headers
+            tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=dev)
+    keys = [f"f{t}" for t in range(T)]
+    kjts = []
+    for _ in range(4):
+        lengths = torch.randint(0, 41, (T * B,), dtype=torch.int32, generator=gen)
+        n = int(lengths.sum())
+        values = torch.randint(0, rows, (n,), dtype=torch.int32, generator=gen).to(dev)
+        weights = torch.rand(n, generator=gen).to(dev)
+        if from_lengths:
+            kjts.append(KeyedJaggedTensor(keys=keys, values=values, weights=weights, lengths=lengths.to(dev)))
+        else:
+            offsets = torch.zeros(T * B + 1, dtype=torch.int32)
+            offsets[1:] = torch.cumsum(lengths, 0)
+            kjts.append(KeyedJaggedTensor(keys=keys, values=values, weights=weights, offsets=offsets.to(dev)))
+    alone = [m(k).values().clone() for k in kjts]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    got = []
+    for k in range(48):
+        with torch.cuda.stream(streams[k % 3]):
+            got.append(m(kjts[k % 4]).values())
+    torch.cuda.synchronize()
+    for k, g in enumerate(got):
+        assert torch.equal(g.view(torch.int16), alone[k % 4].view(torch.int16)), k
+    assert all(t.out_of_range_count() == 0 for t in m._emb_modules)
