@@ -284,3 +284,51 @@ def test_forwards_in_flight_on_several_streams(from_lengths):
     for k, g in enumerate(got):
         assert torch.equal(g.view(torch.int16), alone[k % 4].view(torch.int16)), k
     assert all(t.out_of_range_count() == 0 for t in m._emb_modules)
+
+
+def test_forwards_from_several_host_threads():
+    """Three host threads, each with its own stream, call one module at once
+    (ctypes releases the interpreter lock inside the C entry point)."""
+    import threading
+
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    T, B, rows = 6, 512, 5_000
+    tables = [EmbeddingBagConfig(name=f"t{t}", embedding_dim=32, num_embeddings=rows, feature_names=[f"f{t}"],
+                                 data_type=DataType.INT8, pooling=PoolingType.MEAN) for t in range(T)]
+    m = QuantEBC(tables, False, DEV, output_dtype=torch.float)
+    for tbe in m._emb_modules:
+        tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, generator=gen).to(DEV))
+        for t in range(len(tbe.rows)):
+            tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+    keys = [f"f{t}" for t in range(T)]
+    kjts = []
+    for _ in range(3):
+        lengths = torch.randint(0, 30, (T * B,), dtype=torch.int32, generator=gen)
+        values = torch.randint(0, rows, (int(lengths.sum()),), dtype=torch.int64, generator=gen).to(DEV)
+        kjts.append(KeyedJaggedTensor(keys=keys, values=values, lengths=lengths.to(DEV)))
+    alone = [m(k).values().clone() for k in kjts]
+    torch.cuda.synchronize()
+    results, errors = [None] * 3, []
+
+    def worker(i):
+        try:
+            torch.cuda.set_device(DEV)
+            s = torch.cuda.Stream()
+            outs = []
+            with torch.cuda.stream(s):
+                for k in range(16):
+                    outs.append(m(kjts[(i + k) % 3]).values())
+            s.synchronize()
+            results[i] = outs
+        except Exception as e:  # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(3):
+        for k, o in enumerate(results[i]):
+            assert torch.equal(o, alone[(i + k) % 3]), (i, k)
