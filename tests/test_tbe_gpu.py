@@ -570,6 +570,56 @@ def test_forward_from_lengths_long_prefix(B, idt):
     assert b"from_lengths" in buf.value
 
 
+@pytest.mark.parametrize("seed", range(64))
+def test_random_plans(monkeypatch, seed):
+    """Seeded random operators (table count, weight types, dims, rows, shared and
+    shuffled features, pooling, weights, id and output types, row alignment,
+    pruned ids) through a random route (static kernel, window kernel with a
+    random window, lengths entry) against the oracle, bit for bit."""
+    rng = np.random.default_rng(9000 + seed)
+    T = int(rng.integers(1, 11))
+    pooling = [O.SUM, O.MEAN, O.NONE][int(rng.choice(3, p=[0.45, 0.35, 0.2]))]
+    dims_pool = [16, 32, 48, 64, 96, 128, 160, 256, 320, 512]
+    one_dim = dims_pool[int(rng.integers(0, len(dims_pool)))]
+    specs = []
+    for _ in range(T):
+        dt = [O.INT8, O.INT4, O.INT2, O.FP16, O.FP32][int(rng.integers(0, 5))]
+        dim = one_dim if pooling == O.NONE else dims_pool[int(rng.integers(0, len(dims_pool)))]
+        rows = int(rng.choice([1, 2, 37, 500, 3000]))
+        specs.append((dt, rows, dim))
+    ftm = list(range(T)) + [int(x) for x in rng.integers(0, T, int(rng.integers(0, 4)))]
+    rng.shuffle(ftm)
+    out_dtype = [O.FP32, O.FP16][int(rng.integers(0, 2))]
+    ra = int(rng.choice([4, 8, 16, 64]))
+    idt = [np.int32, np.int64][int(rng.integers(0, 2))]
+    B = int(rng.choice([1, 7, 64, 257, 1500]))
+    max_len = int(rng.choice([1, 3, 20, 70]))
+    weighted = pooling != O.NONE and bool(rng.integers(0, 2))
+    route = ["static", "window", "lengths"][int(rng.integers(0, 3))]
+    window = int(rng.choice([0, 64, 100, 300, 2048]))
+    if route != "static":
+        monkeypatch.setenv("TRA_BALANCED", "1")
+        monkeypatch.setenv("TRA_WINDOW", str(window))
+    else:
+        monkeypatch.setenv("TRA_BALANCED", "0")
+    tbe, store = build(rng, specs, ftm, pooling, out_dtype, ra)
+    rows_f = [specs[t][1] for t in ftm]
+    lengths, offsets, ids = make_bags(rng, rows_f, B, max_len, idt, empty_frac=float(rng.choice([0.0, 0.1, 0.6])))
+    if len(ids) and pooling != O.NONE:
+        ids[rng.random(len(ids)) < 0.05] = -1  # pruned ids are skipped
+    psw = rng.uniform(-2, 2, len(ids)).astype(np.float32) if weighted else None
+    want = O.tbe_forward(store, ftm, B, ids, offsets, psw, pooling, out_dtype)
+    tag = (seed, T, pooling, specs, ftm, out_dtype, ra, idt.__name__, B, max_len, weighted, route, window)
+    if route == "lengths":
+        got = _from_lengths(tbe, ids, lengths, psw, B)
+    else:
+        got = tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV),
+                  None if psw is None else torch.from_numpy(psw).to(DEV)).cpu().numpy()
+    assert got.shape == want.shape, tag
+    assert bits_equal(got, want) == 0, tag
+    assert tbe.out_of_range_count() == 0, tag
+
+
 def test_table_beyond_2_31_rows():
     """A table with more than 2^31 rows (fp32, dim 1: 8.6 GB): int64 ids beyond 2^31 address the
     right rows; int32 ids see every non-negative id as in range; ids >= rows are skipped and counted."""
