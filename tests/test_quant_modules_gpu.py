@@ -332,3 +332,68 @@ def test_forwards_from_several_host_threads():
     for i in range(3):
         for k, o in enumerate(results[i]):
             assert torch.equal(o, alone[(i + k) % 3]), (i, k)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_collections(seed):
+    """Seeded random QuantEmbeddingBagCollections: tables of random type, width
+    and pooling (one lookup operator per pooling), one to three features per
+    table drawn from a small pool (so features are shared between tables and
+    take the feature@table names), a KJT whose keys are a shuffled superset.
+    Output keys follow the reference's naming rule; values match the oracle on
+    the module's own packed bytes, bit for bit."""
+    rng = np.random.default_rng(4000 + seed)
+    pool = [f"f{i}" for i in range(6)]
+    T = int(rng.integers(1, 9))
+    weighted = bool(rng.integers(0, 2))
+    out_dtype = [torch.float, torch.half][int(rng.integers(0, 2))]
+    tables = []
+    for t in range(T):
+        names = [str(x) for x in rng.choice(pool, int(rng.integers(1, 4)), replace=False)]
+        tables.append(EmbeddingBagConfig(
+            name=f"t{t}", embedding_dim=int(rng.choice([16, 32, 64, 128, 192])),
+            num_embeddings=int(rng.choice([3, 40, 700])), feature_names=names,
+            data_type=[DataType.INT8, DataType.INT4, DataType.INT2, DataType.FP16][int(rng.integers(0, 4))],
+            pooling=[PoolingType.SUM, PoolingType.MEAN][int(rng.integers(0, 2))]))
+    m = QuantEBC(tables, weighted, DEV, output_dtype=out_dtype)
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    for tbe in m._emb_modules:
+        tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, generator=gen).to(DEV))
+        for t, ty in enumerate(tbe.weight_tys):
+            if str(ty) in ("int8", "int4", "int2"):  # finite fp16 scale / bias
+                tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+            else:                                    # finite fp16 payload: clear the top exponent bit
+                tbe._rows_view(t)[:, 1::2] &= 0xBF
+    used = sorted({f for t in tables for f in t.feature_names})
+    keys = used + ["unused_a", "unused_b"][: int(rng.integers(0, 3))]
+    rng.shuffle(keys)
+    rows_of = {k: min([t.num_embeddings for t in tables if k in t.feature_names], default=5) for k in keys}
+    B = int(rng.choice([1, 5, 64, 300]))
+    kjt = random_kjt(rng, keys, [rows_of[k] for k in keys], B=B, max_len=int(rng.choice([2, 9, 30])),
+                     weighted=weighted, idt=[torch.int32, torch.int64][int(rng.integers(0, 2))])
+    got = m(kjt)
+    # naming rule (torchrec/modules/embedding_modules.py:75-94): a feature of
+    # several tables is named feature@table; order = tables grouped by pooling
+    count = {f: sum(f in t.feature_names for t in tables) for f in used}
+    grouped = [t for p in (PoolingType.SUM, PoolingType.MEAN) for t in tables if t.pooling == p]
+    if tables[0].pooling == PoolingType.MEAN:  # groups appear in order of first use
+        grouped = [t for p in (PoolingType.MEAN, PoolingType.SUM) for t in tables if t.pooling == p]
+    want_keys = [f if count[f] == 1 else f"{f}@{t.name}" for t in grouped for f in t.feature_names]
+    assert got.keys() == want_keys
+    assert got.length_per_key() == [t.embedding_dim for t in grouped for _ in t.feature_names]
+    order = [kjt.keys().index(k) for k in m._feature_names]
+    perm = kjt.permute(order)
+    ids, offs = perm.values().cpu().numpy(), perm.offsets().cpu().numpy().astype(np.int64)
+    psw = perm.weights().cpu().numpy() if weighted else None
+    col, f0 = 0, 0
+    gv = got.values().cpu().numpy()
+    assert gv.shape == (B, sum(got.length_per_key()))
+    for tbe, nf in zip(m._emb_modules, m._feature_splits):
+        o = offs[f0 * B:(f0 + nf) * B + 1]
+        sl = slice(int(o[0]), int(o[-1]))
+        want = O.tbe_forward(oracle_store_of(tbe), tbe.feature_table_map, B, ids[sl].astype(np.int64), o - o[0],
+                             None if psw is None else psw[sl], int(tbe.pooling_mode),
+                             O.FP16 if out_dtype == torch.half else O.FP32)
+        assert bits_equal(np.ascontiguousarray(gv[:, col:col + tbe.total_D]), want) == 0, (seed, col)
+        col += tbe.total_D
+        f0 += nf
