@@ -397,3 +397,72 @@ def test_random_collections(seed):
         assert bits_equal(np.ascontiguousarray(gv[:, col:col + tbe.total_D]), want) == 0, (seed, col)
         col += tbe.total_D
         f0 += nf
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_sequence_collections(seed):
+    """Seeded random QuantEmbeddingCollections (one lookup operator per weight
+    type, shared features, shuffled superset of keys, need_indices): every
+    output JaggedTensor carries its key's lengths and, row by row, the
+    dequantized rows of the oracle on the module's own packed bytes."""
+    rng = np.random.default_rng(6000 + seed)
+    pool = [f"f{i}" for i in range(5)]
+    T = int(rng.integers(1, 7))
+    dim = int(rng.choice([16, 32, 64, 128]))
+    need_indices = bool(rng.integers(0, 2))
+    out_dtype = [torch.float, torch.half][int(rng.integers(0, 2))]
+    tables = []
+    for t in range(T):
+        names = [str(x) for x in rng.choice(pool, int(rng.integers(1, 3)), replace=False)]
+        tables.append(EmbeddingConfig(
+            name=f"t{t}", embedding_dim=dim, num_embeddings=int(rng.choice([3, 40, 700])), feature_names=names,
+            data_type=[DataType.INT8, DataType.INT4, DataType.INT2, DataType.FP16][int(rng.integers(0, 4))]))
+    m = QuantEC(tables, DEV, need_indices=need_indices, output_dtype=out_dtype)
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    for tbe in m._emb_modules:
+        tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, generator=gen).to(DEV))
+        for t, ty in enumerate(tbe.weight_tys):
+            if str(ty) in ("int8", "int4", "int2"):
+                tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+            else:
+                tbe._rows_view(t)[:, 1::2] &= 0xBF
+    used = sorted({f for t in tables for f in t.feature_names})
+    keys = used + ["unused_a", "unused_b"][: int(rng.integers(0, 3))]
+    rng.shuffle(keys)
+    rows_of = {k: min([t.num_embeddings for t in tables if k in t.feature_names], default=5) for k in keys}
+    B = int(rng.choice([1, 5, 64, 300]))
+    kjt = random_kjt(rng, keys, [rows_of[k] for k in keys], B=B, max_len=int(rng.choice([2, 9, 30])),
+                     idt=[torch.int32, torch.int64][int(rng.integers(0, 2))])
+    got = m(kjt)
+    # Output names are made per lookup operator (torchrec/quant/embedding_modules.py:872-877):
+    # a feature is named feature@table only where it is shared INSIDE its
+    # weight-type group; the same plain name from two groups lands on one
+    # dict entry and the later group's tensor stays.
+    jd = kjt.to_dict()
+    expected = {}
+    f = 0
+    for tbe, nf in zip(m._emb_modules, m._feature_splits):
+        group_features = m._feature_names[f:f + nf]
+        for k in range(nf):
+            feature = group_features[k]
+            t = tbe.feature_table_map[k]
+            name = feature if group_features.count(feature) == 1 else f"{feature}@{tbe.embedding_names[t]}"
+            expected[name] = (tbe, t, feature)
+        f += nf
+    assert set(got.keys()) == set(expected)
+    for name, (tbe, t, feature) in expected.items():
+        jt = got[name]
+        ids = jd[feature].values().cpu().numpy()
+        want = O.tbe_forward(oracle_store_of(tbe), [t], 1, ids, np.array([0, len(ids)], dtype=ids.dtype), None,
+                             O.NONE, O.FP16 if out_dtype == torch.half else O.FP32)
+        assert jt.values().dtype == out_dtype
+        assert bits_equal(jt.values().cpu().numpy(), want) == 0, (seed, name)
+        assert torch.equal(jt.lengths(), jd[feature].lengths())
+        if need_indices:
+            assert torch.equal(jt.weights(), jd[feature].values())
+        else:
+            assert jt.weights_or_none() is None
+    # the accessor names tables over the whole collection (:879-881)
+    count = {f_: sum(f_ in t.feature_names for t in tables) for f_ in used}
+    assert m.embedding_names_by_table() == [
+        [f_ if count[f_] == 1 else f"{f_}@{t.name}" for f_ in t.feature_names] for t in tables]
