@@ -466,3 +466,28 @@ def test_random_sequence_collections(seed):
     count = {f_: sum(f_ in t.feature_names for t in tables) for f_ in used}
     assert m.embedding_names_by_table() == [
         [f_ if count[f_] == 1 else f"{f_}@{t.name}" for f_ in t.feature_names] for t in tables]
+
+
+def test_deepcopy_of_a_used_collection():
+    """A collection that has already looked up (and so holds launch plans) can
+    be deep-copied; the copy has its own bytes and gives the same outputs."""
+    import copy
+
+    rng = np.random.default_rng(21)
+    tables = [EmbeddingBagConfig(name=f"t{i}", embedding_dim=32, num_embeddings=60, feature_names=[f"f{i}"],
+                                 data_type=DataType.INT4) for i in range(3)]
+    m = QuantEBC(tables, False, DEV, output_dtype=torch.float)
+    for tbe in m._emb_modules:
+        tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8).to(DEV))
+        for t in range(len(tbe.rows)):
+            tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+    kjt = random_kjt(rng, ["f0", "f1", "f2"], [60] * 3, B=17, max_len=6)
+    before = m(kjt).values().clone()
+    twin = copy.deepcopy(m)
+    assert torch.equal(twin(kjt).values(), before)
+    twin._emb_modules[0].weights_dev.zero_()
+    assert torch.equal(m(kjt).values(), before)           # the original kept its bytes
+    assert not torch.equal(twin(kjt).values(), before)
+    # the copy's state_dict tensors view the copy's buffer, as the original's view the original's
+    sd = twin.state_dict()
+    assert all(not v.view(torch.uint8).any() for k, v in sd.items() if k.endswith(".weight"))

@@ -193,3 +193,29 @@ def test_operator_follows_its_buffer_between_devices():
     assert op.current_device.type == "meta" and op.weights_dev.device.type == "meta"
     with pytest.raises(_lib.TorchrecAmdError, match="MI355X"):
         op(torch.zeros(2, dtype=torch.int32), torch.tensor([0, 2], dtype=torch.int32))
+
+
+def test_operator_copies_and_pickles_without_its_plans():
+    """Launch plans are C handles owned by one object: a deep copy or a pickle
+    carries the packed bytes and configuration and starts with no plans."""
+    import copy
+    import ctypes
+    import io
+
+    from torchrec_amd.tbe.split_table_batched_embeddings_ops_inference import IntNBitTableBatchedEmbeddingBagsCodegen
+
+    op = IntNBitTableBatchedEmbeddingBagsCodegen(
+        [("t", 10, 8, SparseType.INT8, None)], device=CPU, pooling_mode=PoolingMode.SUM
+    )
+    op.initialize_weights()
+    op.weights_dev.fill_(7)
+    op._plans[None] = ctypes.c_void_p(0)  # stands in for a plan handle (NULL: destroy is a no-op)
+    twin = copy.deepcopy(op)
+    assert twin._plans == {} and len(op._plans) == 1
+    assert torch.equal(twin.weights_dev, op.weights_dev) and twin.weights_dev.data_ptr() != op.weights_dev.data_ptr()
+    buf = io.BytesIO()
+    torch.save(op, buf)
+    buf.seek(0)
+    back = torch.load(buf, weights_only=False)
+    assert back._plans == {} and torch.equal(back.weights_dev, op.weights_dev)
+    assert back.embedding_specs == op.embedding_specs and back.row_bytes == op.row_bytes

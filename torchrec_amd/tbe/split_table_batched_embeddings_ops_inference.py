@@ -252,6 +252,15 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
     def __del__(self) -> None:
         self._drop_plan()
 
+    def __getstate__(self):  # type: ignore[no-untyped-def]
+        """Copies (``copy.deepcopy``) and pickles carry the packed buffer and the
+        configuration; launch plans and scratch buffers belong to this object
+        and are made again on the copy's first lookup."""
+        state = self.__dict__.copy()
+        state["_plans"] = {}
+        state["_workspace"] = {}
+        return state
+
     def _get_plan(self, feature_positions: Optional[Tuple[int, ...]] = None) -> ctypes.c_void_p:
         """Launch plan for one placement of the features among the input keys
         (None: feature f is the f-th key).  Plans are cached per placement."""
