@@ -98,7 +98,9 @@ int tra_tbe_destroy(tra_tbe_t tbe);
  *   out          device; pooled: [B, out_stride] elements, feature f at column
  *                D_offsets[f]; TRA_POOL_NONE: [L, dim] (all features share dim)
  *   out_dtype    TRA_FP32 or TRA_FP16
- *   num_indices  L, the number of elements of indices (required)
+ *   num_indices  L, the number of elements of indices (required); it may
+ *                exceed what the bags cover (a padded buffer): the excess is
+ *                never read
  * Arithmetic per output column, ids in order: acc = fmaf(w*scale, q, acc +
  * w*bias) (fp16/fp32 rows: acc = fmaf(w, x, acc)); MEAN multiplies by 1.0f/len;
  * output rounded to nearest even.  Ids outside [0, rows) other than -1 are

@@ -548,6 +548,31 @@ def test_forward_from_lengths_at_scale():
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+@pytest.mark.parametrize("route", ["static", "window", "lengths"])
+def test_padded_id_buffer(monkeypatch, route):
+    """An id buffer longer than the bags describe (a fixed-size serving buffer
+    with a padded tail): the excess is never looked up, as with the
+    reference's offsets, whichever entry and kernel runs."""
+    monkeypatch.setenv("TRA_BALANCED", "0" if route == "static" else "1")
+    rng = np.random.default_rng(31)
+    rows, B, dim = 2000, 300, 64
+    specs = [(O.INT4, rows, dim), (O.INT8, rows, dim)]
+    tbe, store = build(rng, specs, [0, 1], O.SUM, O.FP32, 16)
+    lengths, offsets, ids = make_bags(rng, [rows, rows], B, 25)
+    psw = rng.uniform(-1, 1, len(ids)).astype(np.float32)
+    want = O.tbe_forward(store, [0, 1], B, ids, offsets, psw, O.SUM, O.FP32)
+    pad = 777
+    ids_p = np.concatenate([ids, np.full(pad, rows + 5, dtype=ids.dtype)])  # the tail would count as out of range
+    psw_p = np.concatenate([psw, np.full(pad, np.float32(np.nan))])
+    if route == "lengths":
+        got = _from_lengths(tbe, ids_p, lengths, psw_p, B)
+    else:
+        got = tbe(torch.from_numpy(ids_p).to(DEV), torch.from_numpy(offsets).to(DEV),
+                  torch.from_numpy(psw_p).to(DEV)).cpu().numpy()
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
+
+
 @pytest.mark.parametrize("B,idt", [(8192, np.int32), (4096, np.int64)])
 def test_forward_from_lengths_long_prefix(B, idt):
     """Enough bags that the blocks of the last windows sum the lengths in front
