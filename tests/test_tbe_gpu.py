@@ -548,6 +548,31 @@ def test_forward_from_lengths_at_scale():
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+@pytest.mark.parametrize("T,B,route", [(1, 70_000, "offsets"), (1, 70_000, "lengths"), (2, 40_000, "lengths"),
+                                       (1, 1_100_000, "offsets"), (1, 1_100_000, "lengths"),
+                                       (300, 3, "offsets"), (300, 3, "lengths"), (300, 40, "lengths"),
+                                       (300, 100, "lengths")])
+def test_extreme_shapes(monkeypatch, T, B, route):
+    """Very tall and very wide calls: a batch beyond what a window entry can
+    index (the static kernel takes over), and hundreds of features with a
+    handful of bags each, through both entries, window kernel requested."""
+    monkeypatch.setenv("TRA_BALANCED", "1")
+    rng = np.random.default_rng(T * 1000 + B)
+    rows, dim = 500, 32
+    dts = [O.INT4, O.INT8, O.FP16]
+    specs = [(dts[t % 3], rows + t, dim) for t in range(T)]
+    ftm = list(range(T))
+    tbe, store = build(rng, specs, ftm, O.MEAN, O.FP16, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * T, B, 6)
+    want = O.tbe_forward(store, ftm, B, ids, offsets, None, O.MEAN, O.FP16)
+    if route == "lengths":
+        got = _from_lengths(tbe, ids, lengths, None, B)
+    else:
+        got = tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV)).cpu().numpy()
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
+
+
 @pytest.mark.parametrize("route", ["static", "window", "lengths"])
 def test_padded_id_buffer(monkeypatch, route):
     """An id buffer longer than the bags describe (a fixed-size serving buffer
