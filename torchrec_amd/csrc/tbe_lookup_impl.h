@@ -679,8 +679,9 @@ struct SumOf<int32_t> { using type = int32_t; };
 // start() adds up every batch but the last and leaves the last one in flight;
 // finish() adds it, so the last round trip overlaps whatever the caller does
 // between the two calls.
-// Every block of the grid reads a prefix of the same array at the same moment,
-// so each starts at a different 16 KB step (`rot`) to spread the L2 channels.
+// Every block of the grid reads a prefix of the same array at the same moment;
+// starting each block at a different 16 KB step to spread the L2 channels
+// measured the same as all starting at the front, so they start at the front.
 // `lengths` is 16-byte aligned.
 constexpr int kPrefixBatch = 8;
 
@@ -691,27 +692,21 @@ struct PrefixSum {
   struct __align__(16) Vec { IdxT v[V]; };
 
   const Vec* vin;
-  int nvec, nk, rot, k_last;
+  int nvec, nk, last, k_last;
   S part;
   IdxT tail;
   Vec x[kPrefixBatch];
 
-  // step k of this block's rotated order (k < nk, rot < nk: one wrap at most)
-  __device__ __forceinline__ int index_of(int k) const {
-    const int j = k + rot;
-    return (j >= nk ? j - nk : j) * kCuThreads + (int)threadIdx.x;
-  }
-  // Always kPrefixBatch loads: were their number to depend on the data, the
-  // compiler could not wait for an older load without draining these.  A step
-  // past the end reads element 0 in every lane (a single request).
+  // Step k of this thread covers vector k * kCuThreads + threadIdx.x; a step
+  // past the end reads the last vector again (clamped) and adds nothing.
   __device__ __forceinline__ Vec fetch(int k) const {
-    return vin[k < nk ? min(index_of(k), nvec - 1) : 0];
+    return vin[min(k * kCuThreads + (int)threadIdx.x, last)];
   }
   __device__ __forceinline__ void add(int k, const Vec& v) {
     S sum = 0;
 #pragma unroll
     for (int i = 0; i < V; ++i) sum += (S)v.v[i];
-    part += (k < nk && index_of(k) < nvec) ? sum : (S)0;
+    part += k * kCuThreads + (int)threadIdx.x < nvec ? sum : (S)0;
   }
   __device__ __forceinline__ void issue(int k0) {
 #pragma unroll
@@ -721,11 +716,11 @@ struct PrefixSum {
 #pragma unroll
     for (int k = 0; k < kPrefixBatch; ++k) add(k0 + k, x[k]);
   }
-  __device__ __forceinline__ void start(const IdxT* __restrict__ lengths, int64_t p, int rot_) {
+  __device__ __forceinline__ void start(const IdxT* __restrict__ lengths, int64_t p) {
     vin = reinterpret_cast<const Vec*>(lengths);
     nvec = (int)(p / V);
     nk = (nvec + kCuThreads - 1) / kCuThreads;
-    rot = nk > 0 ? rot_ % nk : 0;
+    last = max(nvec - 1, 0);
     part = 0;
     // the elements after the last whole 16-byte step: one per lane, clamped like the rest
     const int64_t rest = p - (int64_t)nvec * V;
@@ -857,7 +852,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   PrefixSum<IdxT> front_sum;
   if (FROM_LENGTHS)
     front_sum.start(reinterpret_cast<const IdxT*>(a.offsets),
-                    (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B), blk);
+                    (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B));
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
   lds_barrier();
   TRA_STAMP(6);
@@ -936,7 +931,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
         const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * a.B + (q0 + first - fi * a.B);
         if (fi != fi_lo && pos != next_pos) {
           PrefixSum<IdxT> again;
-          again.start(reinterpret_cast<const IdxT*>(a.offsets), pos, blk);
+          again.start(reinterpret_cast<const IdxT*>(a.offsets), pos);
           const Sum w_ = wave_last(wave_scan_incl(again.finish()));
           if (ln == 0) s_red[wv] = w_;
           lds_barrier();
