@@ -66,6 +66,18 @@ const char* tra_last_error(void);
  * if there is no usable GPU. */
 int tra_device_arch(char* buf, int buf_len);
 
+/* Tuning override for experiments and tests: name is one of "balanced" (1:
+ * window kernel, 0: static kernel), "window" (bags per block), "unroll", "lds",
+ * "xcd" (0: no remap of blocks to dies), "cost_floor", "fused_scan" (from-lengths
+ * prologue inside the lookup kernel: 1 always, 0 never), "cb" (lane chunk bytes,
+ * acts on plans created afterwards); value < 0 restores the default.  The
+ * same knobs are read from the environment (TRA_BALANCED, TRA_WINDOW, ...)
+ * once, when the library is loaded; no lookup call reads the environment.
+ * Process-wide; not meant to be changed while lookups are being issued.
+ * No counterpart in the reference (fbgemm_gpu chooses its kernels internally,
+ * behind the call at torchrec/quant/embedding_modules.py:547-557). */
+int tra_set_tuning(const char* name, int32_t value);
+
 /* TBE group plan ---------------------------------------------------------- */
 /* Builds the immutable launch plan of one TBE group on the current device:
  * per-feature descriptors (feature f reads table feature_table_map[f] and

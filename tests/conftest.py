@@ -25,3 +25,20 @@ def _announce(request):
     if request.node.get_closest_marker("gpu") is not None:
         print(f"\n[gpu-case] {request.node.nodeid}", flush=True)
     yield
+
+
+@pytest.fixture
+def tuning():
+    """Setter of the library's tuning overrides (tra_set_tuning); every knob goes
+    back to its default when the test ends."""
+    from torchrec_amd import _lib
+
+    touched = set()
+
+    def set_(**knobs):
+        touched.update(knobs)
+        _lib.set_tuning(**knobs)
+
+    yield set_
+    if touched:
+        _lib.set_tuning(**{k: None for k in touched})

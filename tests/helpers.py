@@ -55,3 +55,30 @@ def bits_equal(a: np.ndarray, b: np.ndarray) -> int:
     assert a.shape == b.shape and a.dtype == b.dtype, (a.shape, b.shape, a.dtype, b.dtype)
     v = np.uint16 if a.dtype == np.float16 else np.uint32
     return int((a.view(v) != b.view(v)).sum())
+
+
+def bucketize_python(lengths, ids, weights, block_sizes, W, keep):
+    """Independent pure-Python statement of block bucketization (the same rule as
+    block_bucketize_ref in the reference's torchrec/distributed/tests/test_utils.py:299-466)."""
+    F = len(block_sizes)
+    n = len(lengths)
+    B = n // F
+    buckets = [[[] for _ in range(n)] for _ in range(W)]
+    unb = [-1] * len(ids)
+    j = 0
+    for i in range(n):
+        bs = block_sizes[i // B]
+        for _ in range(lengths[i]):
+            p = ids[j] // bs
+            if p < W:
+                buckets[p][i].append((ids[j] if keep else ids[j] % bs, None if weights is None else weights[j], j))
+            j += 1
+    new_l, new_i, new_w = [], [], []
+    for p in range(W):
+        for i in range(n):
+            new_l.append(len(buckets[p][i]))
+            for v, w, src in buckets[p][i]:
+                unb[src] = len(new_i)
+                new_i.append(v)
+                new_w.append(w)
+    return new_l, new_i, new_w, unb

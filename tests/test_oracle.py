@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import oracle as O
-from helpers import bits_equal
+from helpers import bits_equal, bucketize_python
 
 
 def _rows(rng, dim, n=400, bits=4):
@@ -209,3 +209,45 @@ def test_index_math_oracles():
     assert pw.tolist() == [1.5, 1.0, 0.5, 1.0, 0.5, 1.0, 1.0, 1.5]
     pl, pv, _ = O.permute_2d([1, 0, 2, 1, 1], lengths, values)
     assert pv.tolist() == [3.0, 4.0, 5.0, 1.0, 2.0, 6.0, 7.0, 8.0, 3.0, 4.0, 5.0, 3.0, 4.0, 5.0]
+
+
+def test_bucketize_oracle_hand_case():
+    """oracle_bucketize on a case small enough to do by hand: 2 features x 2
+    samples, 2 buckets, block sizes 3 and 5; the id 9 of feature 0 lies beyond
+    the last bucket (9 // 3 = 3 >= 2) and is dropped."""
+    lengths = np.array([2, 1, 1, 2], dtype=np.int64)         # bags (f0,b0) (f0,b1) (f1,b0) (f1,b1)
+    ids = np.array([4, 1, 9, 7, 2, 5], dtype=np.int64)       # f0: [4 1] [9]   f1: [7] [2 5]
+    w = np.array([.1, .2, .3, .4, .5, .6], dtype=np.float32)
+    # bucket of each id: 4//3=1, 1//3=0, 9//3=3 (dropped), 7//5=1, 2//5=0, 5//5=1
+    nl, ni, nw, perm = O.bucketize(lengths, ids, [3, 5], 2, w, False, return_permute=True)
+    assert nl.tolist() == [1, 0, 0, 1,   1, 0, 1, 1]         # bucket-major: [W, F, B]
+    assert ni.tolist() == [1, 2,   1, 2, 0]                  # id % block size, input order inside a bag
+    assert nw.tolist() == [np.float32(x) for x in (.2, .5, .1, .4, .6)]
+    assert perm.tolist() == [2, 0, -1, 3, 1, 4]              # where each input id went; -1 = dropped
+    nl2, ni2, _, _ = O.bucketize(lengths, ids, [3, 5], 2, w, True, return_permute=True)
+    assert nl2.tolist() == nl.tolist() and ni2.tolist() == [1, 2, 4, 7, 5]  # keep_orig_idx: ids as given
+
+
+@pytest.mark.parametrize("F,B,W", [(1, 1, 1), (2, 3, 2), (4, 15, 5), (15, 15, 129), (3, 200, 8)])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+@pytest.mark.parametrize("keep", [False, True])
+def test_bucketize_oracle_matches_python_rule(F, B, W, idt, keep):
+    """oracle_bucketize against an independent pure-Python statement of the rule
+    (the rule of block_bucketize_ref, torchrec/distributed/tests/test_utils.py:379-466):
+    new lengths, new ids, weights and the unbucketize permute, with ids beyond the
+    last bucket dropped, with and without keep_orig_idx."""
+    rng = np.random.default_rng(F * 100 + B * 10 + W)
+    lengths = rng.integers(0, 6, F * B).astype(idt)
+    block_sizes = rng.integers(1, 50, F).astype(np.int64)
+    hi = np.repeat(block_sizes * (W + 1), B)  # some ids fall beyond the last bucket
+    ids = (np.concatenate([rng.integers(0, hi[i], lengths[i]) for i in range(F * B)]).astype(idt)
+           if lengths.sum() else np.zeros(0, idt))
+    weights = rng.random(len(ids)).astype(np.float32)
+    pl, pi, pw, pu = bucketize_python(lengths.tolist(), ids.tolist(), weights.tolist(), block_sizes.tolist(), W, keep)
+    ol, oi, ow, ou = O.bucketize(lengths, ids, block_sizes, W, weights, keep, return_permute=True)
+    assert ol.tolist() == pl and oi.tolist() == pi and ou.tolist() == pu
+    assert np.array_equal(ow, np.asarray(pw, dtype=np.float32))
+    assert (np.asarray(pu) == -1).sum() == len(ids) - len(pi)  # exactly the dropped ids have no place
+    # without weights / without the permute the other outputs do not change
+    ol2, oi2, ow2, ou2 = O.bucketize(lengths, ids, block_sizes, W, None, keep)
+    assert ol2.tolist() == pl and oi2.tolist() == pi and ow2 is None and ou2 is None

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 import oracle as O
+from helpers import bucketize_python
 from torchrec_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -71,33 +72,6 @@ def test_permute_2d(T, B, Tp, idt, vdt, weighted):
         assert gw is None
 
 
-def _bucketize_python(lengths, ids, weights, block_sizes, W, keep):
-    """Independent pure-Python statement of block bucketization (the same rule as
-    block_bucketize_ref in the reference's torchrec/distributed/tests/test_utils.py:299-466)."""
-    F = len(block_sizes)
-    n = len(lengths)
-    B = n // F
-    buckets = [[[] for _ in range(n)] for _ in range(W)]
-    unb = [-1] * len(ids)
-    j = 0
-    for i in range(n):
-        bs = block_sizes[i // B]
-        for _ in range(lengths[i]):
-            p = ids[j] // bs
-            if p < W:
-                buckets[p][i].append((ids[j] if keep else ids[j] % bs, None if weights is None else weights[j], j))
-            j += 1
-    new_l, new_i, new_w = [], [], []
-    for p in range(W):
-        for i in range(n):
-            new_l.append(len(buckets[p][i]))
-            for v, w, src in buckets[p][i]:
-                unb[src] = len(new_i)
-                new_i.append(v)
-                new_w.append(w)
-    return new_l, new_i, new_w, unb
-
-
 @pytest.mark.parametrize("F,B,W", [(1, 1, 1), (2, 3, 2), (4, 15, 5), (15, 15, 129), (3, 200, 8)])
 @pytest.mark.parametrize("idt", [np.int32, np.int64])
 @pytest.mark.parametrize("keep", [False, True])
@@ -109,7 +83,7 @@ def test_bucketize(F, B, W, idt, keep):
     hi = np.repeat(block_sizes * (W + 1), B)
     ids = np.concatenate([rng.integers(0, hi[i], lengths[i]) for i in range(F * B)]).astype(idt) if lengths.sum() else np.zeros(0, idt)
     weights = rng.random(len(ids)).astype(np.float32)
-    pl, pi, pw, pu = _bucketize_python(lengths.tolist(), ids.tolist(), weights.tolist(), block_sizes.tolist(), W, keep)
+    pl, pi, pw, pu = bucketize_python(lengths.tolist(), ids.tolist(), weights.tolist(), block_sizes.tolist(), W, keep)
     ol, oi, ow, ou = O.bucketize(lengths, ids, block_sizes, W, weights, keep, return_permute=True)
     assert ol.tolist() == pl and oi.tolist() == pi and ou.tolist() == pu  # oracle pinned by the python rule
     gl, gi, gw, _, gu = ops.block_bucketize_sparse_features(

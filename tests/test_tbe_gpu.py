@@ -245,20 +245,20 @@ def test_sequence_properties_at_scale():
 
 # The pooled lookup has two kernels: a static bag->wave mapping for small calls
 # and a per-CU window kernel that ranks bags by length (taken when a call has
-# at least 10240 bags and 163840 ids).  TRA_BALANCED / TRA_WINDOW are the
-# library's tuning overrides; the tests below use them to put oracle-sized
-# inputs through the window kernel.
+# at least 10240 bags and 163840 ids).  The library's tuning overrides
+# (tra_set_tuning: "balanced", "window") put oracle-sized inputs through the
+# window kernel in the tests below; the `tuning` fixture restores the defaults.
 
 @pytest.mark.parametrize("dtype", [O.INT8, O.INT4, O.INT2, O.FP16, O.FP32])
 @pytest.mark.parametrize("pooling,weighted", [(O.SUM, False), (O.SUM, True), (O.MEAN, False), (O.MEAN, True)])
-def test_window_kernel_bit_exact(monkeypatch, dtype, pooling, weighted):
+def test_window_kernel_bit_exact(tuning, dtype, pooling, weighted):
     """Window kernel vs oracle: every weight type x pooling, both id widths and
     output types, several windows per feature and a ragged last window."""
-    monkeypatch.setenv("TRA_BALANCED", "1")
+    tuning(balanced=1)
     rng = np.random.default_rng(900 + dtype * 10 + pooling + weighted)
     for dim, out_dtype, idt, window in ((128, O.FP32, np.int32, 64), (64, O.FP16, np.int64, 100),
                                         (256, O.FP16, np.int32, 0), (32, O.FP32, np.int64, 2048)):
-        monkeypatch.setenv("TRA_WINDOW", str(window))
+        tuning(window=window)
         rows, B = 3000, 211
         specs = [(dtype, rows, dim), (dtype, rows + 13, dim)]
         ftm = [0, 1, 0]
@@ -270,13 +270,13 @@ def test_window_kernel_bit_exact(monkeypatch, dtype, pooling, weighted):
         assert tbe.out_of_range_count() == 0
 
 
-def test_window_kernel_mixed_and_edges(monkeypatch):
+def test_window_kernel_mixed_and_edges(tuning):
     """Window kernel: one group mixing weight types and dims (several launch
     classes and sub-classes), bags longer than the exact length bins, empty
     bags, -1 and out-of-range ids, and a key order that differs from the
     operator's feature order."""
-    monkeypatch.setenv("TRA_BALANCED", "1")
-    monkeypatch.setenv("TRA_WINDOW", "96")
+    tuning(balanced=1)
+    tuning(window=96)
     rng = np.random.default_rng(41)
     specs = [([O.INT8, O.INT4, O.INT2, O.FP16][(t // 4) % 4], 500 + 7 * t, [32, 64, 128, 256][t % 4]) for t in range(16)]
     ftm = list(range(16))
@@ -330,7 +330,117 @@ def test_window_kernel_mixed_and_edges(monkeypatch):
     assert (got[:, :dim] == 7.0).all() and (got[:, 3 * dim:] == 7.0).all()
 
 
-def test_window_kernel_equals_static_at_scale(monkeypatch):
+def _position_psw(lens, table, key_start, key_len, B):
+    """Per-id weights the position-weighted entry applies: the id at place k of a
+    bag of key p gets table[key_start[p] + min(k, key_len[p] - 1)]."""
+    out = []
+    for bag, n in enumerate(lens):
+        p = bag // B
+        k = np.minimum(np.arange(n), key_len[p] - 1)
+        out.append(table[key_start[p] + k])
+    return np.concatenate(out).astype(np.float32) if out else np.zeros(0, np.float32)
+
+
+def _run_entry(tbe, entry, ids, lens, offsets, B, table=None, key_start=None, key_len=None):
+    ti = torch.from_numpy(ids).to(DEV)
+    kw = {}
+    if entry.startswith("position"):
+        kw["position_weights"] = (torch.from_numpy(table).to(DEV), list(key_start), list(key_len))
+    if entry in ("lengths", "position_lengths"):
+        return tbe(ti, None, lengths=torch.from_numpy(lens.astype(ids.dtype)).to(DEV), batch_size=B, **kw).cpu().numpy()
+    return tbe(ti, torch.from_numpy(offsets).to(DEV), batch_size=B, **kw).cpu().numpy()
+
+
+LONG_BAG_CASES = {
+    # two bags that share the sort bin 192..255 and meet in one round, the shorter first
+    "200_250": lambda rng, n: _with(rng, n, {0: 200, 1: 250, 9: 255, 10: 192, 17: 254, 30: 193}),
+    # the open last bin (>= 4224)
+    "last_bin": lambda rng, n: _with(rng, n, {2: 4300, 3: 6000, 40: 4224, 41: 9000}),
+    # every bag long, lengths spread over several 64-wide bins
+    "random_150_600": lambda rng, n: rng.integers(150, 601, n),
+    # 64-wide bins 256..319 and 320..383 with many members each
+    "bins_256_383": lambda rng, n: rng.integers(256, 384, n),
+}
+
+
+def _with(rng, n, fixed):
+    lens = rng.integers(0, 12, n)
+    for i, v in fixed.items():
+        lens[i] = v
+    return lens
+
+
+@pytest.mark.parametrize("entry", ["offsets", "lengths", "position_offsets", "position_lengths"])
+@pytest.mark.parametrize("pooling", [O.SUM, O.MEAN])
+@pytest.mark.parametrize("case", sorted(LONG_BAG_CASES))
+def test_window_kernel_long_bags(tuning, entry, pooling, case):
+    """Bags of 192 ids and more, whose sort bins hold a range of lengths, several
+    of them in one window and one round of the window kernel: every id of every
+    bag is pooled (the reference pools a bag whatever its length,
+    torchrec/quant/embedding_modules.py:547-557).  Offsets, lengths and
+    position-weighted entries, SUM and MEAN, against the oracle bit for bit."""
+    tuning(balanced=1, window=128)
+    rng = np.random.default_rng(sum(map(ord, case)) + pooling)
+    rows, dim, B, F = 2000, 128, 48, 2
+    tbe, store = build(rng, [(O.INT4, rows, dim), (O.INT8, rows + 7, dim)], [0, 1], pooling, O.FP32, 16)
+    lens = LONG_BAG_CASES[case](rng, F * B).astype(np.int64)
+    offsets = np.zeros(F * B + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(lens)
+    ids = np.concatenate([rng.integers(0, rows, int(lens[f * B:(f + 1) * B].sum())) for f in range(F)]).astype(np.int32)
+    ids[::11] = -1
+    table = rng.uniform(0.5, 1.5, 40).astype(np.float32)
+    key_start, key_len = [0, 25], [25, 15]
+    psw = _position_psw(lens, table, key_start, key_len, B) if entry.startswith("position") else None
+    want = O.tbe_forward(store, [0, 1], B, ids, offsets, psw, pooling, O.FP32)
+    got = _run_entry(tbe, entry, ids, lens, offsets, B, table, key_start, key_len)
+    assert bits_equal(got, want) == 0, (case, entry, pooling)
+    assert tbe.out_of_range_count() == 0
+
+
+@pytest.mark.parametrize("entry", ["offsets", "lengths"])
+@pytest.mark.parametrize("pooling,weighted", [(O.SUM, False), (O.MEAN, True)])
+def test_long_bags_default_route_at_scale(entry, pooling, weighted):
+    """The same long bags where the window kernel is the default route (12 x
+    1024 bags, lengths 150..600 mixed with short ones, ~1.2 M ids): equal to the
+    static kernel's bits everywhere, and a sample of bags equal to the oracle."""
+    from torchrec_amd import _lib
+    rng = np.random.default_rng(515 + pooling)
+    T, rows, dim, B = 12, 20_000, 128, 1024
+    tbe, store = build(rng, [(O.INT4, rows, dim)] * T, list(range(T)), pooling, O.FP16, 16)
+    lens = rng.integers(0, 30, T * B)
+    long_ = rng.random(T * B) < 0.25
+    lens[long_] = rng.integers(150, 601, int(long_.sum()))
+    offsets = np.zeros(T * B + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(lens)
+    ids = rng.integers(0, rows, int(offsets[-1])).astype(np.int32)
+    psw = rng.uniform(-1, 1, len(ids)).astype(np.float32) if weighted else None
+    ti = torch.from_numpy(ids).to(DEV)
+    tw = None if psw is None else torch.from_numpy(psw).to(DEV)
+    import ctypes
+    buf = ctypes.create_string_buffer(512)
+    _lib.check(_lib.lib().tra_tbe_launch_info(tbe._get_plan(None), B, len(ids), int(tbe.pooling_mode),
+                                              T if entry == "lengths" else 0, buf, 512))
+    assert b"tbe_pooled_cu_kernel" in buf.value
+    if entry == "lengths":
+        a = tbe(ti, None, tw, lengths=torch.from_numpy(lens.astype(np.int32)).to(DEV), batch_size=B)
+    else:
+        a = tbe(ti, torch.from_numpy(offsets).to(DEV), tw)
+    _lib.set_tuning(balanced=0)
+    try:
+        b = tbe(ti, torch.from_numpy(offsets).to(DEV), tw)
+    finally:
+        _lib.set_tuning(balanced=None)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    Bs = 24
+    sub_len = lens.reshape(T, B)[:, :Bs]
+    sub_off = np.zeros(T * Bs + 1, dtype=np.int32)
+    sub_off[1:] = np.cumsum(sub_len.reshape(-1))
+    pick = np.concatenate([np.arange(offsets[f * B], offsets[f * B + Bs]) for f in range(T)])
+    want = O.tbe_forward(store, list(range(T)), Bs, ids[pick], sub_off, None if psw is None else psw[pick], pooling, O.FP16)
+    assert bits_equal(np.ascontiguousarray(a[:Bs].cpu().numpy()), want) == 0
+
+
+def test_window_kernel_equals_static_at_scale(tuning):
     """At a size where the window kernel is the default (26 features x 2048
     samples, ~1M ids) both kernels give the same bits, and a sample of bags
     matches the oracle."""
@@ -341,10 +451,10 @@ def test_window_kernel_equals_static_at_scale(monkeypatch):
     tbe, store = build(rng, specs, ftm, O.SUM, O.FP16, 16)
     lengths, offsets, ids = make_bags(rng, [rows] * T, B, 40, empty_frac=0.02)
     ti, to = torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV)
-    monkeypatch.delenv("TRA_BALANCED", raising=False)
-    monkeypatch.delenv("TRA_WINDOW", raising=False)
+    tuning(balanced=None)
+    tuning(window=None)
     a = tbe(ti, to)
-    monkeypatch.setenv("TRA_BALANCED", "0")
+    tuning(balanced=0)
     b = tbe(ti, to)
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     # oracle on the first 64 samples of every feature
@@ -357,7 +467,7 @@ def test_window_kernel_equals_static_at_scale(monkeypatch):
     assert bits_equal(np.ascontiguousarray(a[:Bs].cpu().numpy()), want) == 0
 
 
-def test_mixed_types_weighted_at_scale(monkeypatch):
+def test_mixed_types_weighted_at_scale(tuning):
     """The mixed workload's shape (weight types and dims mixed, weighted SUM,
     fp32 out, 4096 samples, Poisson(30) bag lengths; 16 tables of 50 K rows):
     several launch classes and sub-classes of the window kernel.  Same bits as
@@ -376,11 +486,11 @@ def test_mixed_types_weighted_at_scale(monkeypatch):
     ids = rng.integers(0, rows, int(offsets[-1])).astype(np.int32)
     psw = rng.uniform(0, 1, len(ids)).astype(np.float32)
     ti, to, tw = (torch.from_numpy(x).to(DEV) for x in (ids, offsets, psw))
-    monkeypatch.delenv("TRA_BALANCED", raising=False)
+    tuning(balanced=None)
     a = tbe(ti, to, tw)
-    monkeypatch.setenv("TRA_BALANCED", "0")
+    tuning(balanced=0)
     b = tbe(ti, to, tw)
-    monkeypatch.delenv("TRA_BALANCED")
+    tuning(balanced=None)
     assert torch.equal(a.view(torch.int32), b.view(torch.int32))
     assert torch.equal(tbe(ti, to, tw * 2), a * 2)
     Bs = 8
@@ -393,14 +503,14 @@ def test_mixed_types_weighted_at_scale(monkeypatch):
 
 
 @pytest.mark.parametrize("from_lengths", [False, True])
-def test_window_kernel_many_features(monkeypatch, from_lengths):
+def test_window_kernel_many_features(tuning, from_lengths):
     """More features than the window kernel keeps close at hand: 300 features
     on three tables (over 128 per launch class: key positions then come from
     the descriptors, not the launch arguments), 3 samples each, 128 bags per
     window (over 32 features per window: their descriptors are read from global
     memory, not from LDS), keys in reverse order."""
-    monkeypatch.setenv("TRA_BALANCED", "1")
-    monkeypatch.setenv("TRA_WINDOW", "128")
+    tuning(balanced=1)
+    tuning(window=128)
     rng = np.random.default_rng(300)
     F, B = 300, 3
     specs = [(O.INT4, 400, 64), (O.INT8, 300, 64), (O.INT4, 500, 32)]
@@ -481,13 +591,13 @@ def _from_lengths(tbe, ids, lengths, psw, B, **kw):
 @pytest.mark.parametrize("dtype,pooling,weighted,idt", [
     (O.INT4, O.SUM, False, np.int32), (O.INT8, O.MEAN, True, np.int64), (O.FP16, O.SUM, True, np.int32),
     (O.INT2, O.MEAN, False, np.int64), (O.FP32, O.SUM, False, np.int32)])
-def test_forward_from_lengths(monkeypatch, window, dtype, pooling, weighted, idt):
+def test_forward_from_lengths(tuning, window, dtype, pooling, weighted, idt):
     """forward(offsets=None, lengths=...) against the oracle: the small-call route
     (scan + lookup, window None) and the window kernel deriving the bag starts
     itself, with windows that span feature boundaries."""
     if window is not None:
-        monkeypatch.setenv("TRA_BALANCED", "1")
-        monkeypatch.setenv("TRA_WINDOW", str(window))
+        tuning(balanced=1)
+        tuning(window=window)
     rng = np.random.default_rng(300 + dtype + pooling + (window or 7))
     rows, B, dim = 3000, 211, 64
     specs = [(dtype, rows, dim), (dtype, rows + 13, dim), (dtype, rows + 5, dim)]
@@ -502,13 +612,13 @@ def test_forward_from_lengths(monkeypatch, window, dtype, pooling, weighted, idt
     assert tbe.out_of_range_count() == 0
 
 
-def test_forward_from_lengths_scattered_keys(monkeypatch):
+def test_forward_from_lengths_scattered_keys(tuning):
     """Window kernel from lengths when the operator's features sit at scattered,
     descending and repeated-gap key positions of a wider KJT (every feature
     boundary inside a window starts a new run), plus an int64 total beyond the
     first features and empty leading keys."""
-    monkeypatch.setenv("TRA_BALANCED", "1")
-    monkeypatch.setenv("TRA_WINDOW", "150")
+    tuning(balanced=1)
+    tuning(window=150)
     rng = np.random.default_rng(17)
     rows, B, dim = 900, 97, 128
     specs = [(O.INT4, rows, dim)] * 4
@@ -552,11 +662,11 @@ def test_forward_from_lengths_at_scale():
                                        (1, 1_100_000, "offsets"), (1, 1_100_000, "lengths"),
                                        (300, 3, "offsets"), (300, 3, "lengths"), (300, 40, "lengths"),
                                        (300, 100, "lengths")])
-def test_extreme_shapes(monkeypatch, T, B, route):
+def test_extreme_shapes(tuning, T, B, route):
     """Very tall and very wide calls: a batch beyond what a window entry can
     index (the static kernel takes over), and hundreds of features with a
     handful of bags each, through both entries, window kernel requested."""
-    monkeypatch.setenv("TRA_BALANCED", "1")
+    tuning(balanced=1)
     rng = np.random.default_rng(T * 1000 + B)
     rows, dim = 500, 32
     dts = [O.INT4, O.INT8, O.FP16]
@@ -574,11 +684,11 @@ def test_extreme_shapes(monkeypatch, T, B, route):
 
 
 @pytest.mark.parametrize("route", ["static", "window", "lengths"])
-def test_padded_id_buffer(monkeypatch, route):
+def test_padded_id_buffer(tuning, route):
     """An id buffer longer than the bags describe (a fixed-size serving buffer
     with a padded tail): the excess is never looked up, as with the
     reference's offsets, whichever entry and kernel runs."""
-    monkeypatch.setenv("TRA_BALANCED", "0" if route == "static" else "1")
+    tuning(balanced=0 if route == "static" else 1)
     rng = np.random.default_rng(31)
     rows, B, dim = 2000, 300, 64
     specs = [(O.INT4, rows, dim), (O.INT8, rows, dim)]
@@ -621,7 +731,7 @@ def test_forward_from_lengths_long_prefix(B, idt):
 
 
 @pytest.mark.parametrize("seed", range(64))
-def test_random_plans(monkeypatch, seed):
+def test_random_plans(tuning, seed):
     """Seeded random operators (table count, weight types, dims, rows, shared and
     shuffled features, pooling, weights, id and output types, row alignment,
     pruned ids) through a random route (static kernel, window kernel with a
@@ -643,15 +753,17 @@ def test_random_plans(monkeypatch, seed):
     ra = int(rng.choice([4, 8, 16, 64]))
     idt = [np.int32, np.int64][int(rng.integers(0, 2))]
     B = int(rng.choice([1, 7, 64, 257, 1500]))
-    max_len = int(rng.choice([1, 3, 20, 70]))
+    max_len = int(rng.choice([1, 3, 20, 70, 300, 5000]))
+    if max_len >= 300:  # long bags: fewer of them, so the oracle stays quick
+        B = min(B, 64 if max_len == 300 else 7)
     weighted = pooling != O.NONE and bool(rng.integers(0, 2))
     route = ["static", "window", "lengths"][int(rng.integers(0, 3))]
     window = int(rng.choice([0, 64, 100, 300, 2048]))
     if route != "static":
-        monkeypatch.setenv("TRA_BALANCED", "1")
-        monkeypatch.setenv("TRA_WINDOW", str(window))
+        tuning(balanced=1)
+        tuning(window=window)
     else:
-        monkeypatch.setenv("TRA_BALANCED", "0")
+        tuning(balanced=0)
     tbe, store = build(rng, specs, ftm, pooling, out_dtype, ra)
     rows_f = [specs[t][1] for t in ftm]
     lengths, offsets, ids = make_bags(rng, rows_f, B, max_len, idt, empty_frac=float(rng.choice([0.0, 0.1, 0.6])))
@@ -670,7 +782,7 @@ def test_random_plans(monkeypatch, seed):
     assert tbe.out_of_range_count() == 0, tag
 
 
-def test_table_beyond_2_31_rows():
+def test_table_beyond_2_31_rows(tuning):
     """A table with more than 2^31 rows (fp32, dim 1: 8.6 GB): int64 ids beyond 2^31 address the
     right rows; int32 ids see every non-negative id as in range; ids >= rows are skipped and counted."""
     rows, B = 2**31 + 1000, 4
@@ -692,12 +804,8 @@ def test_table_beyond_2_31_rows():
     assert got == [4.0 + 5.0, 6.0 + 1.0, 3.0, 2.0]
     assert tbe.out_of_range_count() == 1
     # window kernel, same ids (forced)
-    import os
-    os.environ["TRA_BALANCED"] = "1"
-    try:
-        got = tbe(ids, offsets).cpu().view(-1).tolist()
-    finally:
-        del os.environ["TRA_BALANCED"]
+    tuning(balanced=1)
+    got = tbe(ids, offsets).cpu().view(-1).tolist()
     assert got == [4.0 + 5.0, 6.0 + 1.0, 3.0, 2.0]
     assert tbe.out_of_range_count() == 1
     # int32 ids: every non-negative id is a row of this table

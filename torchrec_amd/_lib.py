@@ -21,6 +21,7 @@ EXPORTED_SYMBOLS = [
     "tra_version",
     "tra_last_error",
     "tra_device_arch",
+    "tra_set_tuning",
     "tra_tbe_create",
     "tra_tbe_destroy",
     "tra_tbe_forward",
@@ -89,6 +90,7 @@ def lib() -> ctypes.CDLL:
         l.tra_tbe_forward_lengths_workspace_bytes.argtypes = [i32, i32, i32]
         l.tra_tbe_forward_lengths_workspace_bytes.restype = i64
         l.tra_tbe_forward_lengths.argtypes = [vp, vp, vp, vp, i32, vp, i32, i32, i64, i32, i32, vp, i64, vp, vp]
+        l.tra_set_tuning.argtypes = [ctypes.c_char_p, i32]
         l.tra_tbe_forward_position_weighted.argtypes = [
             vp, vp, vp, vp, i32, i32, vp, i64, ctypes.POINTER(i32), ctypes.POINTER(i32), i32, i32, i64, i32, i32,
             vp, i64, vp, vp,
@@ -125,6 +127,14 @@ def check(rc: int) -> None:
     if rc != TRA_OK:
         msg = lib().tra_last_error().decode("utf-8", "replace")
         raise TorchrecAmdError(f"torchrec_amd error {rc}: {msg}")
+
+
+def set_tuning(**knobs: Optional[int]) -> None:
+    """Tuning overrides of the lookup (``balanced``, ``window``, ``unroll``, ``lds``, ``xcd``,
+    ``cost_floor``, ``fused_scan``, ``cb``); ``None`` restores a knob's default.  For
+    experiments and tests: process-wide, and not to be changed while lookups are in flight."""
+    for name, value in knobs.items():
+        check(lib().tra_set_tuning(name.encode(), -1 if value is None else int(value)))
 
 
 def require_gpu(t: torch.Tensor, what: str) -> None:

@@ -54,6 +54,7 @@ struct LookupArgs {
   int32_t vec_store;  // 1: every lane's output slice is 16-byte aligned
   int32_t out_fp16;
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
+  int32_t xcd_count;    // balanced pooled kernel: XCDs the grid is dealt to
   int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
   // Position weighting (posw != nullptr): the weight of the id at position k of
   // a bag of class feature ci is posw[pw_off[ci] + min(k, pw_len[ci] - 1)], or
@@ -661,8 +662,9 @@ constexpr int kLenBins = 256;
 constexpr int kMaxWinFeat = 32;  // feature descriptors a window keeps in LDS
 
 // Sort key of a bag length: exact below 192, then steps of 64, then one bin.
+// (A negative length, which only a malformed input holds, ranks as empty.)
 __device__ __forceinline__ int length_bin(int len) {
-  return len < 192 ? len : min(kLenBins - 1, 192 + ((len - 192) >> 6));
+  return len < 192 ? max(len, 0) : min(kLenBins - 1, 192 + ((len - 192) >> 6));
 }
 
 // Accumulator of the from-lengths prologue: as wide as the index type (with
@@ -808,7 +810,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   // Block -> (sub-class, window).  Consecutive windows go to the same XCD
   // (blocks are dealt round-robin to the 8 XCDs), so each L2 sees few tables.
   int blk = blockIdx.x;
-  if (a.xcd_blocks > 0) blk = (blk & 7) * a.xcd_blocks + (blk >> 3);
+  if (a.xcd_blocks > 0) blk = (blk % a.xcd_count) * a.xcd_blocks + blk / a.xcd_count;
   int s = 0;
 #pragma unroll
   for (int i = 1; i < kMaxSub; ++i)
@@ -862,7 +864,10 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     const bool first = i == (int)threadIdx.x;
     int len;
     if (FROM_LENGTHS) {
-      len = max(0, (int)(first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag)));
+      // Kept as given: bag starts are the running sum of the lengths as they
+      // are (what a separate cumsum would produce); a negative length only
+      // makes its own bag empty.
+      len = (int)(first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag));
     } else {
       const int64_t st = first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag);
       const int64_t en = first ? (int64_t)first_hi : load_index<IdxT>(a.offsets, bag + 1);
@@ -999,8 +1004,13 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     const int b = (int)(ent & ((1u << kBagBits) - 1));
     const FeatureDesc d = fi - fi_lo < kMaxWinFeat ? s_desc[fi - fi_lo] : a.descs[a.feats[sc.first + fi]];
     const int64_t start = s_start[i];
-    const int len = active ? s_len[i] : 0;
-    const int max_len = s_len[s_order[r * gpw]];  // the round's first bag is its longest
+    const int len = active ? max(s_len[i], 0) : 0;
+    // The round's trip count.  Lengths below 192 have a sort bin each, so
+    // the round's first bag is its longest; from 192 up a bin holds a range of
+    // lengths in arrival order, and the longest of the round is found by
+    // comparing what the lane groups actually hold.
+    int max_len = s_len[s_order[r * gpw]];
+    if (max_len >= 192) max_len = wave_max(len);
 
     RowWalk w;
     w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
@@ -1082,6 +1092,9 @@ struct LaunchClass {
   std::vector<int32_t> feats;  // plan order: sorted by lpr
   std::vector<int32_t> lprs;   // lanes per row of each feature
   int32_t* feats_dev = nullptr;
+  // every slice's first output column is 16-byte aligned for fp16 / fp32 outputs
+  bool cols_aligned_fp16 = true;
+  bool cols_aligned_fp32 = true;
 };
 
 struct LaunchParams {

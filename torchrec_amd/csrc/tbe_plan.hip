@@ -1,10 +1,13 @@
 // Host side of the TBE lookup: plan construction (tra_tbe_create) and launch
 // (tra_tbe_forward), plus the small library-level entry points.
 #include <algorithm>
+#include <atomic>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <memory>
+#include <mutex>
 #include <string>
 
 #include "tbe_lookup_impl.h"
@@ -37,9 +40,12 @@ int launch_lookup<TRA_FP16>(const LookupArgs&, int, const LaunchParams&, hipStre
 template <>
 int launch_lookup<TRA_FP32>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 
-// Launch shape of the pooled kernels.  Defaults are chosen per call from the
-// problem size; TRA_BALANCED / TRA_WINDOW / TRA_UNROLL / TRA_LDS override them
-// (tuning).
+// Launch shape of the pooled kernels.  Defaults are chosen from the problem
+// size when a plan first sees a (batch size, route) pair and are remembered in
+// the plan.  The tuning overrides (environment TRA_BALANCED, TRA_WINDOW,
+// TRA_UNROLL, TRA_LDS, TRA_XCD, TRA_COST_FLOOR, TRA_FUSED_SCAN, TRA_CB) are read
+// once, when the library is loaded; tra_set_tuning changes them afterwards
+// (experiments and tests).  A forward never reads the environment.
 struct Tuning {
   int balanced;  // 1: tbe_pooled_cu_kernel, one block per CU-sized window of bags
   int window;    // bags per block (0: derive from the problem size)
@@ -47,25 +53,51 @@ struct Tuning {
   int lds_bytes;
 };
 
+struct Overrides {
+  int balanced = -1;    // -1: decide by size
+  int window = -1;      // <= 0: derive
+  int unroll = -1;
+  int lds = -1;
+  int xcd = -1;         // 0: no XCD remap of the window kernel's blocks
+  int cost_floor = -1;
+  int fused_scan = -1;  // -1: decide by size
+  int cb = -1;          // smaller lane chunks (plan creation)
+};
+
 static int env_int(const char* name, int fallback) {
   const char* v = getenv(name);
   return v && *v ? atoi(v) : fallback;
 }
 
-constexpr int kNumCus = 256;
+static Overrides overrides_from_env() {
+  Overrides o;
+  o.balanced = env_int("TRA_BALANCED", -1);
+  o.window = env_int("TRA_WINDOW", -1);
+  o.unroll = env_int("TRA_UNROLL", -1);
+  o.lds = env_int("TRA_LDS", -1);
+  o.xcd = env_int("TRA_XCD", -1);
+  o.cost_floor = env_int("TRA_COST_FLOOR", -1);
+  o.fused_scan = env_int("TRA_FUSED_SCAN", -1);
+  o.cb = env_int("TRA_CB", -1);
+  return o;
+}
 
-static Tuning choose_tuning(int64_t bags, int64_t num_indices) {
+static Overrides g_ovr = overrides_from_env();
+// Bumped by tra_set_tuning: launch geometry remembered under an older value is recomputed.
+static std::atomic<int> g_ovr_gen{0};
+
+static Tuning choose_tuning(int num_cus, int64_t bags, int64_t num_indices) {
   Tuning t;
   // Ranking bags by length pays once every CU gets a few dozen bags (measured
   // crossover on 26 int4 tables: between 6.6k bags / 130k ids and 13k / 260k).
-  t.balanced = bags >= 40 * kNumCus && num_indices >= 640 * (int64_t)kNumCus;
+  t.balanced = bags >= 40 * (int64_t)num_cus && num_indices >= 640 * (int64_t)num_cus;
   t.window = 0;
   t.unroll = 4;
   t.lds_bytes = 48 * 1024;  // with the static arrays > half of a CU's LDS: one block per CU
-  t.balanced = env_int("TRA_BALANCED", t.balanced);
-  t.window = env_int("TRA_WINDOW", t.window);
-  t.unroll = env_int("TRA_UNROLL", t.unroll);
-  t.lds_bytes = env_int("TRA_LDS", t.lds_bytes);
+  if (g_ovr.balanced >= 0) t.balanced = g_ovr.balanced;
+  if (g_ovr.window >= 0) t.window = g_ovr.window;
+  if (g_ovr.unroll >= 0) t.unroll = g_ovr.unroll;
+  if (g_ovr.lds >= 0) t.lds_bytes = g_ovr.lds;
   if (t.window > kMaxWindow) t.window = kMaxWindow;
   if (t.window < 0) t.window = 0;
   return t;
@@ -75,16 +107,47 @@ static Tuning choose_tuning(int64_t bags, int64_t num_indices) {
 
 using namespace tra;
 
+// Launch geometry of one launch class for one (batch size, route).
+struct ClassGeometry {
+  SubClass sub[kMaxSub];
+  int n_sub = 0;
+  int grid = 0;
+  int xcd_blocks = 0;
+  int xcd_count = 1;
+};
+
+// What a plan remembers about a call shape it has seen: the route and, per
+// launch class, the grid and windows.  Recomputed when the tuning overrides change.
+struct Geometry {
+  int32_t batch_size = -1;
+  int64_t nobag_indices = -1;  // sequence lookups size their grid by the id count
+  int balanced = 0;
+  int nobag = 0;
+  int gen = -1;
+  Tuning tune{};
+  std::vector<ClassGeometry> cls;
+};
+
+constexpr int kGeometrySlots = 8;
+
 struct tra_tbe {
   int device = 0;
+  int num_cus = 256;  // compute units of the device (hipDeviceProp_t::multiProcessorCount)
+  int num_xcd = 8;    // accelerator dies, each with its own L2 (hipDeviceAttributeNumberOfXccs)
   int num_features = 0;
   bool same_dim = true;  // every feature has the same dim (required for POOL_NONE)
   int dim0 = 0;
+  int max_key_pos = 0;          // largest feature position among the input keys
+  size_t max_class_feats = 0;   // features of the largest launch class
   std::vector<FeatureDesc> slices;  // host copy
   FeatureDesc* slices_dev = nullptr;
   int32_t* feats_dev = nullptr;  // all classes' slice lists, concatenated
   unsigned long long* err_dev = nullptr;
   std::vector<LaunchClass> classes;
+  std::vector<LookupArgs> base_args;  // per class: everything a call does not change
+  std::mutex geo_mutex;
+  std::shared_ptr<const Geometry> geo[kGeometrySlots];
+  int geo_next = 0;
 };
 
 extern "C" {
@@ -112,6 +175,25 @@ int tra_device_arch(char* buf, int buf_len) {
     return TRA_ERR_NO_DEVICE;
   }
   return TRA_OK;
+}
+
+int tra_set_tuning(const char* name, int32_t value) {
+  if (!name) {
+    set_error("tra_set_tuning: null name");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  struct { const char* n; int* v; } const knobs[] = {
+      {"balanced", &g_ovr.balanced}, {"window", &g_ovr.window}, {"unroll", &g_ovr.unroll},
+      {"lds", &g_ovr.lds}, {"xcd", &g_ovr.xcd}, {"cost_floor", &g_ovr.cost_floor},
+      {"fused_scan", &g_ovr.fused_scan}, {"cb", &g_ovr.cb}};
+  for (const auto& k : knobs)
+    if (strcmp(name, k.n) == 0) {
+      *k.v = value < 0 ? -1 : value;
+      g_ovr_gen.fetch_add(1, std::memory_order_relaxed);
+      return TRA_OK;
+    }
+  set_error("tra_set_tuning: unknown knob '%s'", name);
+  return TRA_ERR_INVALID_ARGUMENT;
 }
 
 int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
@@ -171,7 +253,7 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     // the all-64-byte one).
     int cb = payload % 16 == 0 && payload > 64 ? 16 : (payload % 8 == 0 ? 8 : 4);
     {
-      const int force = env_int("TRA_CB", 0);  // tuning: smaller lane chunks
+      const int force = g_ovr.cb;  // tuning: smaller lane chunks
       if ((force == 8 || force == 4) && force < cb && payload % force == 0) cb = force;
     }
     const int max_slice = cb * kWaveSize;  // bytes one wave-wide lane group covers
@@ -220,6 +302,28 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     flush();
   }
   hipError_t e = hipGetDevice(&plan->device);
+  if (e == hipSuccess) {
+    // The window kernel sizes its grid by the CU count and keeps consecutive
+    // windows on one die: both come from the device, so a partitioned GPU
+    // (fewer CUs, fewer dies) gets a launch that fits it.
+    int cus = 0, xcds = 0;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, plan->device);
+    if (e == hipSuccess && hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, plan->device) != hipSuccess) {
+      (void)hipGetLastError();
+      xcds = 1;
+    }
+    if (e == hipSuccess) {
+      if (cus < 1) {
+        delete plan;
+        set_error("tra_tbe_create: device reports %d compute units", cus);
+        return TRA_ERR_NO_DEVICE;
+      }
+      plan->num_cus = cus;
+      // Blocks are dealt to the dies round-robin; the remap assumes every die
+      // has the same number of CUs.  Anything else: no remap.
+      plan->num_xcd = (xcds >= 1 && cus % xcds == 0) ? xcds : 1;
+    }
+  }
   size_t total = 0;
   for (auto& c : plan->classes) total += c.feats.size();
   if (e == hipSuccess && !plan->slices.empty()) {
@@ -245,6 +349,22 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     tra_tbe_destroy(plan);
     return hip_fail(e, "tra_tbe_create");
   }
+  for (const FeatureDesc& d : plan->slices) plan->max_key_pos = std::max(plan->max_key_pos, (int)d.feature);
+  for (LaunchClass& cls : plan->classes) {
+    for (int id : cls.feats) {
+      cls.cols_aligned_fp16 = cls.cols_aligned_fp16 && (int64_t)plan->slices[id].out_col * 2 % 16 == 0;
+      cls.cols_aligned_fp32 = cls.cols_aligned_fp32 && (int64_t)plan->slices[id].out_col * 4 % 16 == 0;
+    }
+    plan->max_class_feats = std::max(plan->max_class_feats, cls.feats.size());
+    LookupArgs a;
+    memset(&a, 0, sizeof(a));
+    a.descs = plan->slices_dev;
+    a.feats = cls.feats_dev;
+    a.err_count = plan->err_dev;
+    for (size_t i = 0; i < cls.feats.size() && i < (size_t)kMaxPos; ++i)
+      a.feat_pos[i] = (int16_t)plan->slices[cls.feats[i]].feature;
+    plan->base_args.push_back(a);
+  }
   *out = plan;
   return TRA_OK;
 }
@@ -262,14 +382,9 @@ int tra_tbe_destroy(tra_tbe_t tbe) {
 // (or its override) and the limits of the kernel's packed window entries.
 static bool use_window_kernel(const tra_tbe* tbe, const Tuning& tune, bool nobag,
                               int32_t batch_size) {
-  bool balanced = !nobag && tune.balanced && batch_size <= (1 << kBagBits);
-  for (const FeatureDesc& d : tbe->slices)
-    if (d.feature > 32767) balanced = false;
-  for (const LaunchClass& cls : tbe->classes)
-    if ((int64_t)cls.feats.size() >= (int64_t(1) << (32 - kBagBits)) ||
-        (int64_t)cls.feats.size() * batch_size >= (int64_t(1) << 31))
-      balanced = false;
-  return balanced;
+  return !nobag && tune.balanced && batch_size <= (1 << kBagBits) && tbe->max_key_pos <= 32767 &&
+         (int64_t)tbe->max_class_feats < (int64_t(1) << (32 - kBagBits)) &&
+         (int64_t)tbe->max_class_feats * batch_size < (int64_t(1) << 31);
 }
 
 // Largest number of features one window of the from-lengths kernel may span.
@@ -281,9 +396,9 @@ static bool fused_scan_possible(const tra_tbe* tbe, int32_t batch_size, int32_t 
                                 int64_t num_indices, int32_t pooling_mode, const void* lengths) {
   if (pooling_mode == TRA_POOL_NONE || batch_size <= 0 || tbe->num_features == 0) return false;
   if ((uintptr_t)lengths % 16 != 0) return false;
-  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
+  const Tuning tune = choose_tuning(tbe->num_cus, (int64_t)tbe->num_features * batch_size, num_indices);
   if (!use_window_kernel(tbe, tune, false, batch_size)) return false;
-  const int fused = env_int("TRA_FUSED_SCAN", -1);
+  const int fused = g_ovr.fused_scan;
   if (fused >= 0) return fused != 0;
   // A window of up to kMaxWindow bags spans kMaxWindow / B + 2 features at most.
   if (kMaxWindow / batch_size + 2 > kMaxWindowFeatures) return false;
@@ -302,7 +417,7 @@ int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
     return TRA_ERR_INVALID_ARGUMENT;
   }
   const bool nobag = pooling_mode == TRA_POOL_NONE;
-  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
+  const Tuning tune = choose_tuning(tbe->num_cus, (int64_t)tbe->num_features * batch_size, num_indices);
   const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
   // lengths entry point: same decision as tra_tbe_forward_lengths (aligned lengths assumed)
   const bool fused = lengths_num_keys > 0 &&
@@ -332,6 +447,102 @@ struct PositionWeights {
   const int32_t* key_len;
   int32_t num_keys;
 };
+
+// Grid and windows of every launch class for one call shape.
+static void compute_geometry(const tra_tbe* tbe, const Tuning& tune, bool balanced, bool nobag,
+                             int32_t batch_size, int64_t num_indices, Geometry& g) {
+  const int num_cus = tbe->num_cus;
+  g.batch_size = batch_size;
+  g.nobag_indices = nobag ? num_indices : -1;
+  g.balanced = balanced ? 1 : 0;
+  g.nobag = nobag ? 1 : 0;
+  g.tune = tune;
+  g.cls.assign(tbe->classes.size(), ClassGeometry());
+  for (size_t ci = 0; ci < tbe->classes.size(); ++ci) {
+    const LaunchClass& cls = tbe->classes[ci];
+    ClassGeometry& cg = g.cls[ci];
+    // Window kernel: every block should get about the same amount of work, so
+    // a sub-class's window (bags per block) shrinks with its row width.  A
+    // row costs its payload bytes, but never less than 256: below that the
+    // per-row requests (id, header, one line) dominate and rows of any width
+    // take the same time.  Aim at one block per CU; more passes when a window
+    // would not fit the kernel's LDS arrays.
+    const int64_t cost_floor = g_ovr.cost_floor >= 0 ? g_ovr.cost_floor : 256;
+    auto bag_cost = [&](size_t i) { return std::max<int64_t>((int64_t)cls.lprs[i] * cls.cb, cost_floor); };
+    int64_t work_per_block = 0;
+    if (balanced) {
+      int64_t total = 0, min_cost = INT64_MAX;
+      for (size_t i = 0; i < cls.feats.size(); ++i) {
+        total += (int64_t)batch_size * bag_cost(i);
+        min_cost = std::min(min_cost, bag_cost(i));
+      }
+      int64_t blocks = num_cus;
+      while ((total + blocks - 1) / blocks > (int64_t)kMaxWindow * min_cost) blocks += num_cus;
+      work_per_block = (total + blocks - 1) / blocks;
+      // Rounding each sub-class up to whole windows must not spill a few
+      // blocks into an extra pass: grow the share until the grid fits.
+      for (int iter = 0; iter < 64; ++iter) {
+        int64_t grid = 0;
+        for (size_t i = 0; i < cls.feats.size();) {
+          size_t j = i;
+          while (j < cls.feats.size() && cls.lprs[j] == cls.lprs[i]) ++j;
+          const int64_t w = std::max<int64_t>(
+              64, std::min<int64_t>((work_per_block + bag_cost(i) - 1) / bag_cost(i), kMaxWindow));
+          grid += ((int64_t)(j - i) * batch_size + w - 1) / w;
+          i = j;
+        }
+        if (grid <= blocks) break;
+        work_per_block += std::max<int64_t>(1, work_per_block / 128);
+      }
+    }
+    int grid = 0;
+    int n_sub = 0;
+    for (size_t i = 0; i < cls.feats.size();) {
+      size_t j = i;
+      while (j < cls.feats.size() && cls.lprs[j] == cls.lprs[i]) ++j;
+      SubClass& sc = cg.sub[n_sub++];
+      sc.first = (int)i;
+      sc.count = (int)(j - i);
+      sc.lpr = cls.lprs[i];
+      const int gpw = kWaveSize / sc.lpr;
+      const int per_block = kWavesPerBlock * gpw;
+      sc.tile_start = grid;
+      if (nobag) {
+        // Blocks stride over a feature's ids; enough blocks for ~the average
+        // feature, capped so the grid stays modest.
+        int64_t avg = num_indices > 0 ? num_indices / tbe->num_features + 1 : 4096;
+        int64_t t = (avg + per_block - 1) / per_block;
+        sc.tiles_per_feat = (int)std::max<int64_t>(1, std::min<int64_t>(t, 8192));
+        grid += sc.count * sc.tiles_per_feat;
+      } else if (balanced) {
+        const int64_t nb = (int64_t)sc.count * batch_size;
+        int64_t window = tune.window > 0 ? tune.window : (work_per_block + bag_cost(i) - 1) / bag_cost(i);
+        window = std::max<int64_t>(64, std::min<int64_t>(window, kMaxWindow));
+        sc.tiles_per_feat = 0;
+        sc.window = (int)window;
+        grid += (int)((nb + window - 1) / window);
+      } else {
+        sc.tiles_per_feat = (batch_size + per_block - 1) / per_block;
+        grid += sc.count * sc.tiles_per_feat;
+      }
+      i = j;
+    }
+    cg.n_sub = n_sub;
+    cg.grid = grid;
+    cg.xcd_count = 1;
+    cg.xcd_blocks = 0;
+    if (balanced) {
+      // The XCD remap needs a grid that is a whole number of blocks per die
+      // (surplus blocks exit at once).
+      const int nx = tbe->num_xcd;
+      cg.grid = (grid + nx - 1) / nx * nx;
+      if (nx > 1 && g_ovr.xcd != 0) {
+        cg.xcd_blocks = cg.grid / nx;
+        cg.xcd_count = nx;
+      }
+    }
+  }
+}
 
 static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
                         const void* offsets, bool from_lengths, int32_t idx_is_i64,
@@ -390,14 +601,35 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
   }
   const int esz = out_dtype == TRA_FP16 ? 2 : 4;
   hipStream_t s = (hipStream_t)stream;
-  const Tuning tune = choose_tuning((int64_t)tbe->num_features * batch_size, num_indices);
-  const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
-  for (const LaunchClass& cls : tbe->classes) {
-    LookupArgs a;
-    memset(&a, 0, sizeof(a));
+  // Route and launch geometry: remembered per (batch size, route) in the plan.
+  std::shared_ptr<const Geometry> geo;
+  {
+    std::lock_guard<std::mutex> lock(tbe->geo_mutex);
+    const int gen = g_ovr_gen.load(std::memory_order_relaxed);
+    const Tuning tune = choose_tuning(tbe->num_cus, (int64_t)tbe->num_features * batch_size, num_indices);
+    const int balanced = use_window_kernel(tbe, tune, nobag, batch_size) ? 1 : 0;
+    for (const auto& g : tbe->geo)
+      if (g && g->batch_size == batch_size && g->gen == gen && g->balanced == balanced &&
+          g->nobag == (int)nobag && (!nobag || g->nobag_indices == num_indices)) {
+        geo = g;
+        break;
+      }
+    if (!geo) {
+      auto g = std::make_shared<Geometry>();
+      compute_geometry(tbe, tune, balanced != 0, nobag, batch_size, num_indices, *g);
+      g->gen = gen;
+      geo = g;
+      tbe->geo[tbe->geo_next] = geo;  // a call still launching from the replaced entry keeps it alive
+      tbe->geo_next = (tbe->geo_next + 1) % kGeometrySlots;
+    }
+  }
+  const Geometry& geo_local = *geo;
+  const bool balanced = geo_local.balanced != 0;
+  for (size_t ci = 0; ci < tbe->classes.size(); ++ci) {
+    const LaunchClass& cls = tbe->classes[ci];
+    const ClassGeometry& cg = geo_local.cls[ci];
+    LookupArgs a = tbe->base_args[ci];
     a.weights = (const uint8_t*)weights;
-    a.descs = tbe->slices_dev;
-    a.feats = cls.feats_dev;
     // Lanes past the end of their bag still issue (clamped) id loads, so the
     // kernels need one readable element even when there are no ids at all.
     a.indices = num_indices > 0 ? indices : (const void*)tbe->err_dev;
@@ -431,7 +663,6 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     }
     a.out = out;
     a.out_stride = out_stride;
-    a.err_count = tbe->err_dev;
     a.num_indices = num_indices > 0 ? num_indices : 1;
     a.B = batch_size;
     a.mean = pooling_mode == TRA_POOL_MEAN;
@@ -441,90 +672,18 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     if (nobag) {
       vec = vec && ((int64_t)tbe->dim0 * esz % 16 == 0);
     } else {
-      vec = vec && (out_stride * esz % 16 == 0);
+      vec = vec && (out_stride * esz % 16 == 0) && (esz == 2 ? cls.cols_aligned_fp16 : cls.cols_aligned_fp32);
     }
-    if (!nobag)
-      for (int id : cls.feats) vec = vec && ((int64_t)tbe->slices[id].out_col * esz % 16 == 0);
     a.vec_store = vec;
-    // Window kernel: every block should get about the same amount of work, so
-    // a sub-class's window (bags per block) shrinks with its row width.  A
-    // row costs its payload bytes, but never less than 256: below that the
-    // per-row requests (id, header, one line) dominate and rows of any width
-    // take the same time.  Aim at one block per CU; more passes when a window
-    // would not fit the kernel's LDS arrays.
-    const int64_t cost_floor = env_int("TRA_COST_FLOOR", 256);
-    auto bag_cost = [&](size_t i) { return std::max<int64_t>((int64_t)cls.lprs[i] * cls.cb, cost_floor); };
-    int64_t work_per_block = 0;
-    if (balanced) {
-      int64_t total = 0, min_cost = INT64_MAX;
-      for (size_t i = 0; i < cls.feats.size(); ++i) {
-        total += (int64_t)batch_size * bag_cost(i);
-        min_cost = std::min(min_cost, bag_cost(i));
-      }
-      int64_t blocks = kNumCus;
-      while ((total + blocks - 1) / blocks > (int64_t)kMaxWindow * min_cost) blocks += kNumCus;
-      work_per_block = (total + blocks - 1) / blocks;
-      // Rounding each sub-class up to whole windows must not spill a few
-      // blocks into an extra pass: grow the share until the grid fits.
-      for (int iter = 0; iter < 64; ++iter) {
-        int64_t g = 0;
-        for (size_t i = 0; i < cls.feats.size();) {
-          size_t j = i;
-          while (j < cls.feats.size() && cls.lprs[j] == cls.lprs[i]) ++j;
-          const int64_t w = std::max<int64_t>(
-              64, std::min<int64_t>((work_per_block + bag_cost(i) - 1) / bag_cost(i), kMaxWindow));
-          g += ((int64_t)(j - i) * batch_size + w - 1) / w;
-          i = j;
-        }
-        if (g <= blocks) break;
-        work_per_block += std::max<int64_t>(1, work_per_block / 128);
-      }
-      for (size_t i = 0; i < cls.feats.size() && i < (size_t)kMaxPos; ++i)
-        a.feat_pos[i] = (int16_t)tbe->slices[cls.feats[i]].feature;
-    }
-    int grid = 0;
-    int n_sub = 0;
-    for (size_t i = 0; i < cls.feats.size();) {
-      size_t j = i;
-      while (j < cls.feats.size() && cls.lprs[j] == cls.lprs[i]) ++j;
-      SubClass& sc = a.sub[n_sub++];
-      sc.first = (int)i;
-      sc.count = (int)(j - i);
-      sc.lpr = cls.lprs[i];
-      const int gpw = kWaveSize / sc.lpr;
-      const int per_block = kWavesPerBlock * gpw;
-      sc.tile_start = grid;
-      if (nobag) {
-        // Blocks stride over a feature's ids; enough blocks for ~the average
-        // feature, capped so the grid stays modest.
-        int64_t avg = num_indices > 0 ? num_indices / tbe->num_features + 1 : 4096;
-        int64_t t = (avg + per_block - 1) / per_block;
-        sc.tiles_per_feat = (int)std::max<int64_t>(1, std::min<int64_t>(t, 8192));
-        grid += sc.count * sc.tiles_per_feat;
-      } else if (balanced) {
-        const int64_t nb = (int64_t)sc.count * batch_size;
-        int64_t window = tune.window > 0 ? tune.window : (work_per_block + bag_cost(i) - 1) / bag_cost(i);
-        window = std::max<int64_t>(64, std::min<int64_t>(window, kMaxWindow));
-        sc.tiles_per_feat = 0;
-        sc.window = (int)window;
-        grid += (int)((nb + window - 1) / window);
-      } else {
-        sc.tiles_per_feat = (batch_size + per_block - 1) / per_block;
-        grid += sc.count * sc.tiles_per_feat;
-      }
-      i = j;
-    }
-    a.n_sub = n_sub;
+    memcpy(a.sub, cg.sub, sizeof(a.sub));
+    a.n_sub = cg.n_sub;
+    a.xcd_blocks = cg.xcd_blocks;
+    a.xcd_count = cg.xcd_count;
     LaunchParams lp;
     lp.balanced = balanced ? 1 : 0;
-    lp.lds_bytes = tune.lds_bytes;
-    lp.grid = grid;
-    if (balanced) {
-      // XCD remap needs a grid that is a multiple of 8 (surplus blocks exit at once).
-      lp.grid = (grid + 7) / 8 * 8;
-      a.xcd_blocks = env_int("TRA_XCD", 1) ? lp.grid / 8 : 0;
-    }
-    lp.unroll = tune.unroll;
+    lp.lds_bytes = geo_local.tune.lds_bytes;
+    lp.grid = cg.grid;
+    lp.unroll = geo_local.tune.unroll;
     lp.idx64 = idx_is_i64 != 0;
     lp.weighted = a.psw != nullptr || a.posw != nullptr;
     lp.nobag = nobag;
