@@ -146,6 +146,25 @@ int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indi
                             int32_t pooling_mode, int32_t out_dtype, void* out,
                             int64_t out_stride, void* workspace, void* stream);
 
+/* tra_tbe_forward_lengths without a workspace argument and without any
+ * allocation: the scratch (the offsets array and the scan's partial sums, the
+ * same bytes tra_tbe_forward_lengths_workspace_bytes() asks for) lives in a
+ * static device array of the library, tra_tbe_forward_lengths_static_max_bytes()
+ * = 8 MiB per GPU, resolved when the first plan is created on that GPU.  No
+ * counterpart in the reference; it is for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  A call that needs more scratch returns TRA_ERR_TOO_LARGE.
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (several streams or host threads) race; nothing in it has to start at zero.
+ * Results are those of tra_tbe_forward_lengths. */
+int64_t tra_tbe_forward_lengths_static_max_bytes(void);
+int tra_tbe_forward_lengths_static(tra_tbe_t tbe, const void* weights, const void* indices,
+                                   const void* lengths, int32_t idx_is_i64,
+                                   const float* per_sample_weights, int32_t batch_size,
+                                   int32_t num_keys, int64_t num_indices,
+                                   int32_t pooling_mode, int32_t out_dtype, void* out,
+                                   int64_t out_stride, void* stream);
+
 /* Pooled lookup with position weights: the id at position k of a bag of the
  * feature at key position p is weighted by
  *   position_weights[key_start[p] + min(k, key_len[p] - 1)],  or 1 if key_len[p] == 0,

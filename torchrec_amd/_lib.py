@@ -27,6 +27,8 @@ EXPORTED_SYMBOLS = [
     "tra_tbe_forward",
     "tra_tbe_forward_lengths_workspace_bytes",
     "tra_tbe_forward_lengths",
+    "tra_tbe_forward_lengths_static_max_bytes",
+    "tra_tbe_forward_lengths_static",
     "tra_tbe_forward_position_weighted",
     "tra_tbe_launch_info",
     "tra_tbe_error_count",
@@ -90,6 +92,8 @@ def lib() -> ctypes.CDLL:
         l.tra_tbe_forward_lengths_workspace_bytes.argtypes = [i32, i32, i32]
         l.tra_tbe_forward_lengths_workspace_bytes.restype = i64
         l.tra_tbe_forward_lengths.argtypes = [vp, vp, vp, vp, i32, vp, i32, i32, i64, i32, i32, vp, i64, vp, vp]
+        l.tra_tbe_forward_lengths_static_max_bytes.restype = i64
+        l.tra_tbe_forward_lengths_static.argtypes = [vp, vp, vp, vp, i32, vp, i32, i32, i64, i32, i32, vp, i64, vp]
         l.tra_set_tuning.argtypes = [ctypes.c_char_p, i32]
         l.tra_tbe_forward_position_weighted.argtypes = [
             vp, vp, vp, vp, i32, i32, vp, i64, ctypes.POINTER(i32), ctypes.POINTER(i32), i32, i32, i64, i32, i32,

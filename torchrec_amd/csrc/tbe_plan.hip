@@ -105,6 +105,40 @@ static Tuning choose_tuning(int num_cus, int64_t bags, int64_t num_indices) {
 
 }  // namespace tra
 
+// Scratch of tra_tbe_forward_lengths_static: the offsets array and the scan's
+// tile sums of one call.  One copy per GPU, held until the process ends.
+constexpr int64_t kStaticScratchBytes = 8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace tra {
+
+// Device address of `scratch` on each GPU (the array's name is only a host-side
+// handle).  Resolved when the first plan is created on a device, that device
+// being current.
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+static int resolve_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices) {
+    set_error("device index %d is beyond the %d devices the library tracks", device, kMaxDevices);
+    return TRA_ERR_TOO_LARGE;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] != nullptr) return TRA_OK;
+  void* p = nullptr;
+  hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+  if (p == nullptr || (uintptr_t)p % 256 != 0) {
+    set_error("static scratch resolved to %p (expected a 256-byte aligned device address)", p);
+    return TRA_ERR_HIP;
+  }
+  g_scratch_ptr[device] = p;
+  return TRA_OK;
+}
+
+}  // namespace tra
+
 using namespace tra;
 
 // Launch geometry of one launch class for one (batch size, route).
@@ -143,6 +177,7 @@ struct tra_tbe {
   FeatureDesc* slices_dev = nullptr;
   int32_t* feats_dev = nullptr;  // all classes' slice lists, concatenated
   unsigned long long* err_dev = nullptr;
+  void* static_scratch = nullptr;  // this device's copy of the library's static scratch array
   std::vector<LaunchClass> classes;
   std::vector<LookupArgs> base_args;  // per class: everything a call does not change
   std::mutex geo_mutex;
@@ -322,6 +357,12 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
       // Blocks are dealt to the dies round-robin; the remap assumes every die
       // has the same number of CUs.  Anything else: no remap.
       plan->num_xcd = (xcds >= 1 && cus % xcds == 0) ? xcds : 1;
+      const int rc = resolve_static_scratch(plan->device);
+      if (rc != TRA_OK) {
+        delete plan;
+        return rc;
+      }
+      plan->static_scratch = g_scratch_ptr[plan->device];
     }
   }
   size_t total = 0;
@@ -771,6 +812,33 @@ int tra_tbe_forward_lengths(tra_tbe_t tbe, const void* weights, const void* indi
   return forward_lengths_impl(tbe, weights, indices, lengths, idx_is_i64, per_sample_weights,
                               batch_size, num_keys, num_indices, pooling_mode, out_dtype, out,
                               out_stride, workspace, stream, nullptr);
+}
+
+int64_t tra_tbe_forward_lengths_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int tra_tbe_forward_lengths_static(tra_tbe_t tbe, const void* weights, const void* indices,
+                                   const void* lengths, int32_t idx_is_i64,
+                                   const float* per_sample_weights, int32_t batch_size,
+                                   int32_t num_keys, int64_t num_indices, int32_t pooling_mode,
+                                   int32_t out_dtype, void* out, int64_t out_stride, void* stream) {
+  if (!tbe) {
+    set_error("tra_tbe_forward_lengths_static: null plan");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int64_t need = tra_tbe_forward_lengths_workspace_bytes(num_keys, batch_size, idx_is_i64);
+  if (need > kStaticScratchBytes) {
+    set_error("tra_tbe_forward_lengths_static: %d keys x %d samples need %lld bytes of scratch, the static "
+              "buffer holds %lld; use tra_tbe_forward_lengths with a workspace",
+              num_keys, batch_size, (long long)need, (long long)kStaticScratchBytes);
+    return TRA_ERR_TOO_LARGE;
+  }
+  if (!tbe->static_scratch) {
+    set_error("tra_tbe_forward_lengths_static: the static scratch was not resolved for device %d", tbe->device);
+    return TRA_ERR_HIP;
+  }
+  return forward_lengths_impl(tbe, weights, indices, lengths, idx_is_i64, per_sample_weights,
+                              batch_size, num_keys, num_indices, pooling_mode, out_dtype, out,
+                              out_stride, tbe->static_scratch, stream, nullptr);
 }
 
 int tra_tbe_forward_position_weighted(tra_tbe_t tbe, const void* weights, const void* indices,
