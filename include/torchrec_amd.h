@@ -252,7 +252,11 @@ int tra_permute_2d_data(const int32_t* permute, int32_t num_out_features,
  * itself if keep_orig_idx), weights, and optionally unbucketize_permute [L]
  * (output position of each input id, -1 if dropped).  Order inside one
  * (bucket, f, b) is the input order.  offsets is the complete cumsum of
- * lengths; cursor_workspace is device scratch of W*F*B int64. */
+ * lengths; cursor_workspace is device scratch of
+ * tra_bucketize_workspace_bytes() bytes (0 up to 1024 buckets: NULL is then
+ * accepted; W*F*B int64 beyond). */
+int64_t tra_bucketize_workspace_bytes(int32_t num_features, int32_t batch_size,
+                                      int32_t num_buckets);
 int tra_bucketize_lengths(const void* offsets, const void* indices,
                           int32_t is_i64, const int64_t* block_sizes,
                           int32_t num_features, int32_t batch_size,

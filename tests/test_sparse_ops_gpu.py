@@ -149,3 +149,99 @@ def test_quantize_rows_bytes_identical(bits):
         # a host tensor is staged through the GPU and comes back on the host
         got_h = ops.FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(torch.from_numpy(w[:100]), bits)
         assert got_h.device.type == "cpu" and np.array_equal(got_h.numpy(), want[:100])
+
+
+def _lengths_like(kind, n, rng):
+    if kind == "short":
+        ln = rng.integers(0, 41, n)
+        ln[rng.random(n) < 0.05] = 0
+    elif kind == "poisson":
+        ln = rng.poisson(30.0, n)
+    else:  # a few very long bags among empty and short ones: chunks of 64 ids inside one bag
+        ln = rng.integers(0, 4, n)
+        ln[rng.integers(0, n, max(1, n // 500))] = rng.integers(65, 700, max(1, n // 500))
+    return ln
+
+
+@pytest.mark.parametrize("F,B,W,kind", [
+    (26, 2048, 8, "short"),      # 8 bags per wave
+    (64, 4096, 4, "poisson"),    # 64 bags per wave
+    (8, 16384, 16, "long"),
+    (3, 5000, 1, "long"),
+    (5, 1000, 700, "short"),     # one bag per wave (wide bucketization)
+    (2, 300, 1500, "short"),     # beyond the wave kernels' bucket limit: thread-per-bag kernels
+])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+def test_bucketize_at_scale(F, B, W, kind, idt):
+    rng = np.random.default_rng(F * B + W)
+    n = F * B
+    lengths = _lengths_like(kind, n, rng).astype(idt)
+    block_sizes = rng.integers(1000, 200_000, F).astype(np.int64)
+    if idt == np.int64:
+        block_sizes[0] = (1 << 33) + 12345  # 64-bit division
+    L = int(lengths.sum())
+    per_id_bs = np.repeat(np.repeat(block_sizes, B), lengths)
+    top = np.minimum(per_id_bs * (W + 1), np.iinfo(idt).max)  # some ids fall beyond the last bucket
+    ids = (rng.random(L) * top).astype(idt)
+    weights = rng.random(L).astype(np.float32)
+    for keep in (False, True):
+        ol, oi, ow, ou = O.bucketize(lengths, ids, block_sizes, W, weights, keep, return_permute=True)
+        gl, gi, gw, _, gu = ops.block_bucketize_sparse_features(
+            torch.from_numpy(lengths).to(DEV), torch.from_numpy(ids).to(DEV), False, True,
+            torch.from_numpy(block_sizes).to(DEV), W, torch.from_numpy(weights).to(DEV), keep)
+        assert np.array_equal(gl.cpu().numpy(), ol)
+        assert np.array_equal(gi.cpu().numpy(), oi)
+        assert np.array_equal(gu.cpu().numpy(), ou)
+        assert np.array_equal(gw.cpu().numpy(), ow)
+    # what the layout itself fixes: every kept id sits in the bucket its value names, in input order
+    kept = ou >= 0
+    assert int(ol.sum()) == int(kept.sum())
+    assert np.array_equal(oi[ou[kept]], ids[kept])  # (keep=True run is the last one)
+
+
+@pytest.mark.parametrize("F,B,kind", [(26, 2048, "short"), (64, 4096, "poisson"), (8, 16384, "long"), (1, 1, "long"),
+                                      (3, 77, "short")])
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+def test_offsets_range_and_position_weights_at_scale(F, B, kind, idt):
+    rng = np.random.default_rng(F + B)
+    n = F * B
+    lengths = _lengths_like(kind, n, rng).astype(idt)
+    L = int(lengths.sum())
+    offsets = np.zeros(n + 1, dtype=idt)
+    offsets[1:] = np.cumsum(lengths)
+    want_range = (np.arange(L) - np.repeat(offsets[:-1], lengths)).astype(idt)
+    got = ops.offsets_range(torch.from_numpy(offsets[:-1].copy()).to(DEV), L)
+    assert got.dtype == torch.from_numpy(offsets).dtype and np.array_equal(got.cpu().numpy(), want_range)
+    # a range cut short: ids at or beyond range_size are not produced
+    if L > 10:
+        cut = L - 7
+        assert np.array_equal(ops.offsets_range(torch.from_numpy(offsets[:-1].copy()).to(DEV), cut).cpu().numpy(),
+                              want_range[:cut])
+    # position weights: key k has a table of key_len[k] entries (0: no table -> 1.0); positions
+    # beyond the table take its last entry
+    key_len = rng.integers(0, 50, F).astype(np.int32)
+    key_len[rng.integers(0, F)] = 0
+    key_start = np.zeros(F, dtype=np.int32)
+    key_start[1:] = np.cumsum(key_len)[:-1]
+    table = rng.random(max(int(key_len.sum()), 1)).astype(np.float32)
+    key_of_id = np.repeat(np.repeat(np.arange(F), B), lengths)
+    klen = key_len[key_of_id]
+    pos = np.minimum(want_range, np.maximum(klen - 1, 0))
+    want_w = np.where(klen > 0, table[np.minimum(key_start[key_of_id] + pos, len(table) - 1)], np.float32(1.0)).astype(np.float32)
+    got_w = ops.position_weights(torch.from_numpy(offsets).to(DEV), F, B, torch.from_numpy(key_start).to(DEV),
+                                 torch.from_numpy(key_len).to(DEV), torch.from_numpy(table).to(DEV), L)
+    assert np.array_equal(got_w.cpu().numpy(), want_w)
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+def test_quantize_rows_odd_dims(bits):
+    """Dims on either side of the dword-per-lane kernel's alignment rule, rows wider than one wave's
+    worth of dwords, and a row count that leaves the last wave partly idle."""
+    rng = np.random.default_rng(100 + bits)
+    for dim in (4, 12, 20, 40, 96, 200, 520, 2048):
+        if dim % (8 // bits):
+            continue
+        w = rng.normal(0, 1.0, (1237, dim)).astype(np.float32)
+        want = O.quantize_sbhalf(w, bits)
+        got = ops.FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(torch.from_numpy(w).to(DEV), bits).cpu().numpy()
+        assert np.array_equal(got, want), (bits, dim, int((got != want).sum()))

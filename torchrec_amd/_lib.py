@@ -37,6 +37,7 @@ EXPORTED_SYMBOLS = [
     "tra_length_per_key",
     "tra_permute_2d_lengths",
     "tra_permute_2d_data",
+    "tra_bucketize_workspace_bytes",
     "tra_bucketize_lengths",
     "tra_bucketize_scatter",
     "tra_quantize_rows",
@@ -107,6 +108,8 @@ def lib() -> ctypes.CDLL:
         l.tra_length_per_key.argtypes = [vp, i32, i32, i32, vp, vp]
         l.tra_permute_2d_lengths.argtypes = [vp, i32, i32, i32, vp, i32, vp, vp]
         l.tra_permute_2d_data.argtypes = [vp, i32, i32, vp, vp, i32, vp, i32, vp, vp, vp, vp]
+        l.tra_bucketize_workspace_bytes.argtypes = [i32, i32, i32]
+        l.tra_bucketize_workspace_bytes.restype = i64
         l.tra_bucketize_lengths.argtypes = [vp, vp, i32, vp, i32, i32, i32, vp, vp]
         l.tra_bucketize_scatter.argtypes = [vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp]
         l.tra_quantize_rows.argtypes = [vp, i64, i32, i32, vp, i32, vp]

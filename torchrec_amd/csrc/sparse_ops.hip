@@ -250,6 +250,156 @@ __global__ void bucketize_scatter_kernel(const void* offsets, const void* indice
   }
 }
 
+// ---- a wave walking the ids of its own run of bags ---------------------------
+// The id-parallel kernels below (bucketization, positions in bags, position
+// weights) share one mapping: a wave owns `bpw` consecutive bags (a power of
+// two, at most 64), keeps their bounds in LDS and visits their ids in order,
+// 64 at a time, so every load and store of ids is coalesced; the bag of an id
+// is found by a branch-free search over the wave's bounds.  Waves never share
+// LDS, so the only synchronization is program order inside the wave.
+constexpr int kWalkThreads = 256;
+constexpr int kWalkWaves = kWalkThreads / kWaveSize;
+constexpr int kWalkMaxBuckets = 1024;  // wider bucketizations take the thread-per-bag kernels
+
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront", "local");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// Largest b in [0, cnt) with off[b] <= j; off[0] <= j holds.  top_step = bpw / 2.
+__device__ __forceinline__ int find_bag(const int64_t* off, int cnt, int top_step, int64_t j) {
+  int lo = 0;
+  for (int step = top_step; step >= 1; step >>= 1) {
+    const int c = lo + step;
+    if (c < cnt && off[c] <= j) lo = c;
+  }
+  return lo;
+}
+
+// id / bs and id % bs; 32-bit arithmetic where both fit.
+__device__ __forceinline__ void div_mod(uint64_t id, uint64_t bs, uint64_t& q, uint64_t& r) {
+  if (((id | bs) >> 32) == 0) {
+    const uint32_t a = (uint32_t)id, b = (uint32_t)bs;
+    const uint32_t qq = a / b;
+    q = qq;
+    r = a - qq * b;
+  } else {
+    q = id / bs;
+    r = id - q * bs;
+  }
+}
+
+// Bags per wave for n bags: 64, halved while that leaves fewer than 4096
+// waves, and never more than `cap`.
+static int bags_per_wave(int64_t n, int cap) {
+  int bpw = 64;
+  while (bpw > 1 && (bpw > cap || (n + bpw - 1) / bpw < 4096)) bpw >>= 1;
+  return bpw;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWalkThreads) void bucketize_lengths_wave_kernel(
+    const T* __restrict__ offsets, const T* __restrict__ indices, const int64_t* __restrict__ block_sizes,
+    int32_t B, int64_t n, int32_t W, int bpw, T* __restrict__ new_lengths) {
+  extern __shared__ int64_t walk_smem[];
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  const int per_wave = (bpw + 1) + bpw + (W * bpw + 1) / 2;  // int64 units
+  int64_t* s_off = walk_smem + (size_t)wave * per_wave;
+  int64_t* s_bs = s_off + bpw + 1;
+  int32_t* s_cnt = reinterpret_cast<int32_t*>(s_bs + bpw);
+  const int64_t i0 = ((int64_t)blockIdx.x * kWalkWaves + wave) * bpw;
+  if (i0 >= n) return;
+  const int cnt = (int)(n - i0 < bpw ? n - i0 : bpw);
+  for (int k = lane; k <= cnt; k += kWaveSize) s_off[k] = (int64_t)offsets[i0 + k];
+  for (int k = lane; k < cnt; k += kWaveSize) s_bs[k] = block_sizes[(i0 + k) / B];
+  for (int k = lane; k < W * bpw; k += kWaveSize) s_cnt[k] = 0;
+  wave_lds_sync();
+  const int64_t first = s_off[0], last = s_off[cnt];
+  for (int64_t j0 = first; j0 < last; j0 += kWaveSize) {
+    const int64_t j = j0 + lane;
+    if (j < last) {
+      const int64_t id = (int64_t)indices[j];
+      const int b = find_bag(s_off, cnt, bpw >> 1, j);
+      uint64_t q, r;
+      div_mod((uint64_t)id, (uint64_t)s_bs[b], q, r);
+      if (q < (uint64_t)W) atomicAdd(&s_cnt[(int)q * bpw + b], 1);
+    }
+  }
+  wave_lds_sync();
+  for (int x = lane; x < W * cnt; x += kWaveSize) {
+    const int p = x / cnt, k = x - p * cnt;
+    new_lengths[(int64_t)p * n + i0 + k] = (T)s_cnt[p * bpw + k];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kWalkThreads) void bucketize_scatter_wave_kernel(
+    const T* __restrict__ offsets, const T* __restrict__ indices, const float* __restrict__ weights,
+    const int64_t* __restrict__ block_sizes, int32_t B, int64_t n, int32_t W, int bpw, int keep_orig,
+    const T* __restrict__ new_offsets, T* __restrict__ new_indices, float* __restrict__ new_weights,
+    int64_t* __restrict__ unbucketize_permute) {
+  extern __shared__ int64_t walk_smem[];
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  const int per_wave = (bpw + 1) + bpw + W * bpw;
+  int64_t* s_off = walk_smem + (size_t)wave * per_wave;
+  int64_t* s_bs = s_off + bpw + 1;
+  int64_t* s_cur = s_bs + bpw;  // next output position of (bucket p, bag b) at [p * bpw + b]
+  const int64_t i0 = ((int64_t)blockIdx.x * kWalkWaves + wave) * bpw;
+  if (i0 >= n) return;
+  const int cnt = (int)(n - i0 < bpw ? n - i0 : bpw);
+  for (int k = lane; k <= cnt; k += kWaveSize) s_off[k] = (int64_t)offsets[i0 + k];
+  for (int k = lane; k < cnt; k += kWaveSize) s_bs[k] = block_sizes[(i0 + k) / B];
+  for (int x = lane; x < W * cnt; x += kWaveSize) {
+    const int p = x / cnt, k = x - p * cnt;
+    s_cur[p * bpw + k] = (int64_t)new_offsets[(int64_t)p * n + i0 + k];
+  }
+  wave_lds_sync();
+  const int64_t first = s_off[0], last = s_off[cnt];
+  const uint64_t below_me = lane == 0 ? 0ull : (~0ull >> (kWaveSize - lane));
+  for (int64_t j0 = first; j0 < last; j0 += kWaveSize) {
+    const int64_t j = j0 + lane;
+    const bool valid = j < last;
+    const int64_t id = valid ? (int64_t)indices[j] : 0;
+    const int b = find_bag(s_off, cnt, bpw >> 1, valid ? j : first);
+    uint64_t q = 0, r = 0;
+    div_mod((uint64_t)id, (uint64_t)s_bs[b], q, r);
+    const bool in = valid && q < (uint64_t)W;
+    const int p = in ? (int)q : -1;
+    // The lanes of this chunk that hold ids of my bag: [lo_lane, hi_lane).
+    const int64_t lo64 = s_off[b] - j0, hi64 = s_off[b + 1] - j0;
+    const int lo_lane = lo64 < 0 ? 0 : (lo64 > kWaveSize - 1 ? kWaveSize - 1 : (int)lo64);
+    const int hi_lane = hi64 > kWaveSize ? kWaveSize : (hi64 < 0 ? 0 : (int)hi64);
+    const uint64_t my_bag = (hi_lane >= kWaveSize ? ~0ull : ((1ull << hi_lane) - 1)) & ~((1ull << lo_lane) - 1);
+    // Rank of my id among the ids of the same bag and bucket in this chunk
+    // (input order), one pass per bucket value present in the wave.
+    int rank = 0, same_count = 0;
+    uint64_t rem = __builtin_amdgcn_ballot_w64(in);
+    while (rem != 0) {
+      const int leader = __builtin_amdgcn_readfirstlane(__builtin_ctzll(rem));
+      const int pl = __builtin_amdgcn_readlane(p, leader);
+      const uint64_t m = __builtin_amdgcn_ballot_w64(in && p == pl);
+      if (in && p == pl) {
+        const uint64_t same = m & my_bag;
+        rank = __builtin_popcountll(same & below_me);
+        same_count = __builtin_popcountll(same);
+      }
+      rem &= ~m;
+    }
+    int64_t pos = -1;
+    if (in) {
+      pos = s_cur[p * bpw + b] + rank;
+      new_indices[pos] = keep_orig ? (T)id : (T)r;
+      if (weights) new_weights[pos] = weights[j];
+    }
+    if (valid && unbucketize_permute) unbucketize_permute[j] = pos;
+    wave_lds_sync();  // every lane has read its cursor
+    if (in && rank == same_count - 1) s_cur[p * bpw + b] = pos + 1;
+    wave_lds_sync();
+  }
+}
+
 // ---- row-wise N-bit quantization -------------------------------------------
 // One wave per row.  Same operation order as fbgemm's
 // FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf: min/max, bias = fp16(min),
@@ -314,37 +464,149 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* in, int
   }
 }
 
-// ---- positions inside bags ---------------------------------------------------
-// One thread per bag: range[j] = j - start(bag) for the bag's ids.
-template <typename T>
-__global__ void offsets_range_kernel(const void* offsets, int64_t n, int64_t range_size, void* out) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int64_t s = ld<T>(offsets, i);
-  const int64_t e = i + 1 < n ? ld<T>(offsets, i + 1) : range_size;
-  for (int64_t j = s; j < e && j < range_size; ++j) st<T>(out, j, j - s);
+// The same quantizer for rows whose elements and output rows are 4-byte
+// aligned (dim a multiple of 32 / BITS): a lane owns the 32 / BITS consecutive
+// elements of one output dword, loads them 16 bytes at a time and stores the
+// dword whole; `lpr` lanes (a power of two) share a row, 64 / lpr rows a wave.
+// Per element the arithmetic is that of quantize_rows_kernel.
+template <int BITS>
+__global__ __launch_bounds__(256) void quantize_rows_vec_kernel(const float* __restrict__ in, int64_t rows,
+                                                                int32_t dim, uint8_t* __restrict__ out,
+                                                                int64_t row_bytes, int header_first,
+                                                                int lpr) {
+  constexpr int EPL = 32 / BITS;  // elements per output dword
+  constexpr int kQMax = (1 << BITS) - 1;
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int g = lane / lpr, c = lane - g * lpr;
+  const int rows_per_wave = kWaveSize / lpr;
+  const int64_t r_raw = ((int64_t)blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize) * rows_per_wave + g;
+  const bool active = r_raw < rows;
+  const int64_t r = active ? r_raw : rows - 1;  // every lane takes part in the reductions
+  const float* x = in + r * dim;
+  const int chunks = dim / EPL;
+  float mn = x[0], mx = mn;
+  float keep[EPL];  // the lane's first chunk stays in registers for the second pass
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) keep[e] = mn;
+  for (int ch = c; ch < chunks; ch += lpr) {
+    float v[EPL];
+#pragma unroll
+    for (int k = 0; k < EPL / 4; ++k) {
+      const float4 q = *reinterpret_cast<const float4*>(x + ch * EPL + 4 * k);
+      v[4 * k] = q.x; v[4 * k + 1] = q.y; v[4 * k + 2] = q.z; v[4 * k + 3] = q.w;
+    }
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      mn = v[e] < mn ? v[e] : mn;
+      mx = v[e] > mx ? v[e] : mx;
+      if (ch == c) keep[e] = v[e];
+    }
+  }
+  for (int off = lpr >> 1; off > 0; off >>= 1) {
+    const float a = __shfl_xor(mn, off, 64), b = __shfl_xor(mx, off, 64);
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+  }
+  const __half bias_h = __float2half_rn(mn);
+  const float bias = __half2float(bias_h);
+  const float range = mx - bias;
+  float scale = range == 0.0f ? 1.0f : range / (float)kQMax;
+  scale = __half2float(__float2half_rn(scale));
+  if (scale == 0.0f) scale = 1.0f;
+  float inv = 1.0f / scale;
+  if (__builtin_isinf(inv)) {
+    scale = 1.0f;
+    inv = 1.0f;
+  }
+  const __half scale_h = __float2half_rn(scale);
+  if (!active) return;
+  uint8_t* o = out + r * row_bytes;
+  uint32_t* pay = reinterpret_cast<uint32_t*>(header_first ? o + 4 : o);
+  uint32_t* hdr = reinterpret_cast<uint32_t*>(header_first ? o : o + (int64_t)chunks * 4);
+  for (int ch = c; ch < chunks; ch += lpr) {
+    float v[EPL];
+    if (ch == c) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) v[e] = keep[e];
+    } else {
+#pragma unroll
+      for (int k = 0; k < EPL / 4; ++k) {
+        const float4 q = *reinterpret_cast<const float4*>(x + ch * EPL + 4 * k);
+        v[4 * k] = q.x; v[4 * k + 1] = q.y; v[4 * k + 2] = q.z; v[4 * k + 3] = q.w;
+      }
+    }
+    uint32_t packed = 0;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const float t = (v[e] - bias) * inv;
+      float q = __builtin_rintf(t);
+      q = q < 0.0f ? 0.0f : q;
+      q = q > (float)kQMax ? (float)kQMax : q;
+      packed |= (uint32_t)(int)q << (e * BITS);
+    }
+    pay[ch] = packed;
+  }
+  if (c == 0) *hdr = (uint32_t)__half_as_ushort(scale_h) | ((uint32_t)__half_as_ushort(bias_h) << 16);
 }
 
-// One thread per bag of key k: weight[j] = table[key_start[k] + (j - start)],
+// ---- positions inside bags ---------------------------------------------------
+// range[j] = j - start(bag of j), for j < range_size; `offsets` has n entries
+// and the last bag ends at range_size.
+template <typename T>
+__global__ __launch_bounds__(kWalkThreads) void offsets_range_kernel(const T* __restrict__ offsets, int64_t n,
+                                                                      int64_t range_size, int bpw,
+                                                                      T* __restrict__ out) {
+  extern __shared__ int64_t walk_smem[];
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  int64_t* s_off = walk_smem + (size_t)wave * (bpw + 1);
+  const int64_t i0 = ((int64_t)blockIdx.x * kWalkWaves + wave) * bpw;
+  if (i0 >= n) return;
+  const int cnt = (int)(n - i0 < bpw ? n - i0 : bpw);
+  for (int k = lane; k <= cnt; k += kWaveSize) {
+    int64_t v = i0 + k < n ? (int64_t)offsets[i0 + k] : range_size;
+    v = v < 0 ? 0 : v;
+    s_off[k] = v < range_size ? v : range_size;
+  }
+  wave_lds_sync();
+  const int64_t first = s_off[0], last = s_off[cnt];
+  for (int64_t j = first + lane; j < last; j += kWaveSize) {
+    const int b = find_bag(s_off, cnt, bpw >> 1, j);
+    out[j] = (T)(j - s_off[b]);
+  }
+}
+
+// weight[j] = table[key_start[k] + (j - start of j's bag)] for an id of key k,
 // 1.0 for keys without a table.  Positions at or beyond the key's table length
 // take the last entry.
 template <typename T>
-__global__ void position_weights_kernel(const void* offsets, int32_t B, int64_t n,
-                                        const int32_t* key_start, const int32_t* key_len,
-                                        const float* table, float* out) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int k = (int)(i / B);
-  const int64_t s = ld<T>(offsets, i), e = ld<T>(offsets, i + 1);
-  const int len = key_len[k];
-  if (len <= 0) {
-    for (int64_t j = s; j < e; ++j) out[j] = 1.0f;
-    return;
+__global__ __launch_bounds__(kWalkThreads) void position_weights_kernel(
+    const T* __restrict__ offsets, int32_t B, int64_t n, const int32_t* __restrict__ key_start,
+    const int32_t* __restrict__ key_len, const float* __restrict__ table, int bpw, float* __restrict__ out) {
+  extern __shared__ int64_t walk_smem[];
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  int64_t* s_off = walk_smem + (size_t)wave * (2 * bpw + 1);
+  int32_t* s_start = reinterpret_cast<int32_t*>(s_off + bpw + 1);
+  int32_t* s_len = s_start + bpw;
+  const int64_t i0 = ((int64_t)blockIdx.x * kWalkWaves + wave) * bpw;
+  if (i0 >= n) return;
+  const int cnt = (int)(n - i0 < bpw ? n - i0 : bpw);
+  for (int k = lane; k <= cnt; k += kWaveSize) s_off[k] = (int64_t)offsets[i0 + k];
+  for (int k = lane; k < cnt; k += kWaveSize) {
+    const int key = (int)((i0 + k) / B);
+    s_start[k] = key_start[key];
+    s_len[k] = key_len[key];
   }
-  const float* t = table + key_start[k];
-  for (int64_t j = s; j < e; ++j) {
-    const int64_t pos = j - s;
-    out[j] = t[pos < len ? pos : len - 1];
+  wave_lds_sync();
+  const int64_t first = s_off[0], last = s_off[cnt];
+  for (int64_t j = first + lane; j < last; j += kWaveSize) {
+    const int b = find_bag(s_off, cnt, bpw >> 1, j);
+    const int len = s_len[b];
+    const int64_t pos = j - s_off[b];
+    float w = 1.0f;
+    if (len > 0) w = table[s_start[b] + (int)(pos < len ? pos : len - 1)];
+    out[j] = w;
   }
 }
 
@@ -460,6 +722,26 @@ static int quantize_impl(const float* in, int64_t rows, int32_t dim, int32_t bit
   if (!in || !out) {
     set_error("quantize: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
+  }
+  const int epl = 32 / bits;
+  if (dim % epl == 0 && row_bytes % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 4 == 0) {
+    const int chunks = dim / epl;
+    int lpr = 1;
+    while (lpr < chunks && lpr < kWaveSize) lpr <<= 1;
+    const int64_t rows_per_block = 4 * (kWaveSize / lpr);
+    const int64_t vblocks = (rows + rows_per_block - 1) / rows_per_block;
+    if (vblocks > 0x7fffffff) {
+      set_error("quantize: too many rows in one call");
+      return TRA_ERR_TOO_LARGE;
+    }
+    dim3 vg((unsigned)vblocks), vb(256);
+    if (bits == 8)
+      hipLaunchKernelGGL(quantize_rows_vec_kernel<8>, vg, vb, 0, s, in, rows, dim, out, row_bytes, header_first, lpr);
+    else if (bits == 4)
+      hipLaunchKernelGGL(quantize_rows_vec_kernel<4>, vg, vb, 0, s, in, rows, dim, out, row_bytes, header_first, lpr);
+    else
+      hipLaunchKernelGGL(quantize_rows_vec_kernel<2>, vg, vb, 0, s, in, rows, dim, out, row_bytes, header_first, lpr);
+    return check_launch("quantize_rows");
   }
   const int64_t blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffff) {
@@ -632,6 +914,21 @@ int tra_bucketize_lengths(const void* offsets, const void* indices, int32_t is_i
     return TRA_ERR_INVALID_ARGUMENT;
   }
   hipStream_t s = (hipStream_t)stream;
+  if (num_buckets <= kWalkMaxBuckets) {
+    const int bpw = bags_per_wave(n, std::max(1, kWalkMaxBuckets / num_buckets));
+    const int64_t waves = (n + bpw - 1) / bpw;
+    dim3 g((unsigned)((waves + kWalkWaves - 1) / kWalkWaves)), b(kWalkThreads);
+    const size_t lds = (size_t)kWalkWaves * ((bpw + 1) + bpw + ((size_t)num_buckets * bpw + 1) / 2) * sizeof(int64_t);
+    if (is_i64)
+      hipLaunchKernelGGL(bucketize_lengths_wave_kernel<int64_t>, g, b, lds, s, (const int64_t*)offsets,
+                         (const int64_t*)indices, block_sizes, batch_size, n, num_buckets, bpw,
+                         (int64_t*)new_lengths);
+    else
+      hipLaunchKernelGGL(bucketize_lengths_wave_kernel<int32_t>, g, b, lds, s, (const int32_t*)offsets,
+                         (const int32_t*)indices, block_sizes, batch_size, n, num_buckets, bpw,
+                         (int32_t*)new_lengths);
+    return check_launch("tra_bucketize_lengths");
+  }
   dim3 g((unsigned)((n + 127) / 128)), b(128);
   if (is_i64)
     hipLaunchKernelGGL(bucketize_lengths_kernel<int64_t>, g, b, 0, s, offsets, indices, block_sizes,
@@ -640,6 +937,11 @@ int tra_bucketize_lengths(const void* offsets, const void* indices, int32_t is_i
     hipLaunchKernelGGL(bucketize_lengths_kernel<int32_t>, g, b, 0, s, offsets, indices, block_sizes,
                        batch_size, n, num_buckets, new_lengths);
   return check_launch("tra_bucketize_lengths");
+}
+
+int64_t tra_bucketize_workspace_bytes(int32_t num_features, int32_t batch_size, int32_t num_buckets) {
+  if (num_features <= 0 || batch_size <= 0 || num_buckets <= kWalkMaxBuckets) return 0;
+  return (int64_t)num_features * batch_size * num_buckets * (int64_t)sizeof(int64_t);
 }
 
 int tra_bucketize_scatter(const void* offsets, const void* indices, int32_t is_i64,
@@ -653,11 +955,32 @@ int tra_bucketize_scatter(const void* offsets, const void* indices, int32_t is_i
     return TRA_ERR_INVALID_ARGUMENT;
   }
   if (n == 0) return TRA_OK;
-  if (!offsets || !block_sizes || !new_offsets || !cursor_workspace || (weights && !new_weights)) {
+  if (!offsets || !block_sizes || !new_offsets || (weights && !new_weights)) {
     set_error("tra_bucketize_scatter: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
   }
   hipStream_t s = (hipStream_t)stream;
+  if (num_buckets <= kWalkMaxBuckets) {
+    const int bpw = bags_per_wave(n, std::max(1, kWalkMaxBuckets / num_buckets));
+    const int64_t waves = (n + bpw - 1) / bpw;
+    dim3 g((unsigned)((waves + kWalkWaves - 1) / kWalkWaves)), b(kWalkThreads);
+    const size_t lds = (size_t)kWalkWaves * ((bpw + 1) + bpw + (size_t)num_buckets * bpw) * sizeof(int64_t);
+    if (is_i64)
+      hipLaunchKernelGGL(bucketize_scatter_wave_kernel<int64_t>, g, b, lds, s, (const int64_t*)offsets,
+                         (const int64_t*)indices, weights, block_sizes, batch_size, n, num_buckets, bpw,
+                         keep_orig_idx, (const int64_t*)new_offsets, (int64_t*)new_indices, new_weights,
+                         unbucketize_permute);
+    else
+      hipLaunchKernelGGL(bucketize_scatter_wave_kernel<int32_t>, g, b, lds, s, (const int32_t*)offsets,
+                         (const int32_t*)indices, weights, block_sizes, batch_size, n, num_buckets, bpw,
+                         keep_orig_idx, (const int32_t*)new_offsets, (int32_t*)new_indices, new_weights,
+                         unbucketize_permute);
+    return check_launch("tra_bucketize_scatter");
+  }
+  if (!cursor_workspace) {
+    set_error("tra_bucketize_scatter: more than %d buckets need the cursor workspace", kWalkMaxBuckets);
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
   dim3 g((unsigned)((n + 127) / 128)), b(128);
   if (is_i64)
     hipLaunchKernelGGL(bucketize_scatter_kernel<int64_t>, g, b, 0, s, offsets, indices, weights,
@@ -692,13 +1015,16 @@ int tra_offsets_range(const void* offsets, int64_t num_bags, int32_t is_i64, int
     set_error("tra_offsets_range: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
   }
-  dim3 g((unsigned)((num_bags + 127) / 128)), b(128);
+  const int bpw = bags_per_wave(num_bags, 64);
+  const int64_t waves = (num_bags + bpw - 1) / bpw;
+  dim3 g((unsigned)((waves + kWalkWaves - 1) / kWalkWaves)), b(kWalkThreads);
+  const size_t lds = (size_t)kWalkWaves * (bpw + 1) * sizeof(int64_t);
   if (is_i64)
-    hipLaunchKernelGGL(offsets_range_kernel<int64_t>, g, b, 0, (hipStream_t)stream, offsets, num_bags,
-                       range_size, out);
+    hipLaunchKernelGGL(offsets_range_kernel<int64_t>, g, b, lds, (hipStream_t)stream, (const int64_t*)offsets,
+                       num_bags, range_size, bpw, (int64_t*)out);
   else
-    hipLaunchKernelGGL(offsets_range_kernel<int32_t>, g, b, 0, (hipStream_t)stream, offsets, num_bags,
-                       range_size, out);
+    hipLaunchKernelGGL(offsets_range_kernel<int32_t>, g, b, lds, (hipStream_t)stream, (const int32_t*)offsets,
+                       num_bags, range_size, bpw, (int32_t*)out);
   return check_launch("tra_offsets_range");
 }
 
@@ -715,13 +1041,16 @@ int tra_position_weights(const void* offsets, int32_t is_i64, int32_t num_keys, 
     set_error("tra_position_weights: null buffer");
     return TRA_ERR_INVALID_ARGUMENT;
   }
-  dim3 g((unsigned)((n + 127) / 128)), b(128);
+  const int bpw = bags_per_wave(n, 64);
+  const int64_t waves = (n + bpw - 1) / bpw;
+  dim3 g((unsigned)((waves + kWalkWaves - 1) / kWalkWaves)), b(kWalkThreads);
+  const size_t lds = (size_t)kWalkWaves * (2 * bpw + 1) * sizeof(int64_t);
   if (is_i64)
-    hipLaunchKernelGGL(position_weights_kernel<int64_t>, g, b, 0, (hipStream_t)stream, offsets,
-                       batch_size, n, key_start, key_len, table, out);
+    hipLaunchKernelGGL(position_weights_kernel<int64_t>, g, b, lds, (hipStream_t)stream, (const int64_t*)offsets,
+                       batch_size, n, key_start, key_len, table, bpw, out);
   else
-    hipLaunchKernelGGL(position_weights_kernel<int32_t>, g, b, 0, (hipStream_t)stream, offsets,
-                       batch_size, n, key_start, key_len, table, out);
+    hipLaunchKernelGGL(position_weights_kernel<int32_t>, g, b, lds, (hipStream_t)stream, (const int32_t*)offsets,
+                       batch_size, n, key_start, key_len, table, bpw, out);
   return check_launch("tra_position_weights");
 }
 

@@ -194,7 +194,8 @@ def block_bucketize_sparse_features(
     unbucketize = (
         torch.empty(indices.numel(), dtype=torch.int64, device=dev) if sequence else None
     )
-    cursor = torch.empty(max(W * n, 1), dtype=torch.int64, device=dev)
+    ws_bytes = l.tra_bucketize_workspace_bytes(F, B, W)
+    cursor = torch.empty(ws_bytes // 8, dtype=torch.int64, device=dev) if ws_bytes else None
     _lib.check(
         l.tra_bucketize_scatter(
             _lib.ptr(offsets), _lib.ptr(indices), is64, _lib.ptr(weights), _lib.ptr(bs), F, B, W,
