@@ -658,6 +658,52 @@ def test_forward_from_lengths_at_scale():
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
+def _launch_text(tbe, B, n_ids, n_keys):
+    import ctypes
+    from torchrec_amd import _lib
+    buf = ctypes.create_string_buffer(1024)
+    _lib.check(_lib.lib().tra_tbe_launch_info(tbe._get_plan(None), B, n_ids, int(tbe.pooling_mode), n_keys, buf, 1024))
+    return buf.value.decode()
+
+
+@pytest.mark.parametrize("B,idt,pooling,weighted", [
+    (1, np.int32, O.SUM, False), (37, np.int64, O.MEAN, True), (512, np.int32, O.SUM, True),
+    (1170, np.int32, O.MEAN, False), (1171, np.int64, O.SUM, False)])
+def test_small_call_from_lengths_one_launch(tuning, B, idt, pooling, weighted):
+    """A call too small for the window kernel, given lengths: up to 16384 lengths the static kernel sums
+    the lengths in front of each block itself (one launch, no scan kernel); beyond, or with
+    fused_scan=0, a scan runs first.  Both against the oracle, mixed row widths (1 to 32 lanes per
+    row), 12 features at shuffled positions of a 14-key KJT, batch sizes that leave tiles partly empty."""
+    rng = np.random.default_rng(4000 + B)
+    dims = [32, 64, 128, 256, 8, 16]
+    dts = [O.INT8, O.INT4, O.FP16, O.INT2, O.FP32, O.INT8]
+    specs = [(dts[t], 700 + 13 * t, dims[t]) for t in range(6)]
+    ftm = [0, 1, 2, 3, 4, 5, 0, 1, 2, 3, 4, 5]
+    K = 14
+    positions = list(rng.permutation(K)[:12])
+    tbe, store = build(rng, specs, ftm, pooling, O.FP32, 16)
+    # (few enough ids that the call stays with the static kernel at the larger batch sizes)
+    lengths, offsets, ids = make_bags(rng, [700] * K, B, 33 if B < 1000 else 10, idt, empty_frac=0.2)
+    psw = rng.uniform(-1, 1, len(ids)).astype(np.float32) if weighted else None
+    seg = [ids[offsets[k * B]:offsets[(k + 1) * B]] for k in range(K)]
+    wseg = None if psw is None else [psw[offsets[k * B]:offsets[(k + 1) * B]] for k in range(K)]
+    Lm = lengths.reshape(K, B)
+    o_off = np.zeros(12 * B + 1, dtype=idt)
+    o_off[1:] = np.cumsum(np.concatenate([Lm[p] for p in positions]))
+    want = O.tbe_forward(store, ftm, B, np.concatenate([seg[p] for p in positions]), o_off,
+                         None if psw is None else np.concatenate([wseg[p] for p in positions]), pooling, O.FP32)
+    fused_expected = K * B <= 16384
+    text = _launch_text(tbe, B, len(ids), K)
+    assert ("tbe_pooled_kernel" in text) and (("from_lengths" in text) == fused_expected) and (("scan" in text) != fused_expected), text
+    got = _from_lengths(tbe, ids, lengths, psw, B, feature_positions=positions)
+    assert bits_equal(got, want) == 0
+    tuning(fused_scan=0)
+    assert "scan" in _launch_text(tbe, B, len(ids), K)
+    got = _from_lengths(tbe, ids, lengths, psw, B, feature_positions=positions)
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
+
+
 @pytest.mark.parametrize("T,B,route", [(1, 70_000, "offsets"), (1, 70_000, "lengths"), (2, 40_000, "lengths"),
                                        (1, 1_100_000, "offsets"), (1, 1_100_000, "lengths"),
                                        (300, 3, "offsets"), (300, 3, "lengths"), (300, 40, "lengths"),

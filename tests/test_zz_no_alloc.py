@@ -66,14 +66,16 @@ def test_static_scratch_entry_two_calls_in_a_row():
     rows_f = [s[1] for s in specs]
     buf = ctypes.create_string_buffer(512)
     # call 1: 4 x 40000 bags: scan in tiles (partial sums in the scratch), window kernel from offsets
-    # call 2: 4 x 300 bags: one-launch scan, static kernel
-    for B, max_len in ((40_000, 6), (300, 20)):
+    # call 2: 4 x 5000 bags of few ids: one-launch scan into the scratch, static kernel
+    # (a call of at most 16384 lengths would not touch the scratch at all: its one kernel
+    # derives the bag starts itself)
+    for B, max_len in ((40_000, 6), (5000, 5)):
         lengths, offsets, ids = make_bags(rng, rows_f, B, max_len)
         _lib.check(_lib.lib().tra_tbe_launch_info(tbe._get_plan(None), B, len(ids), _lib.POOL_SUM, K, buf, 512))
         assert b"from_lengths" not in buf.value and b"scan" in buf.value, buf.value
         got_static, got_ws = _both_entries(tbe, ids, lengths, B, K, total_D)
         assert bits_equal(got_static, got_ws) == 0, B
-        if B <= 1000:
+        if B <= 5000:
             want = O.tbe_forward(store, list(range(K)), B, ids, offsets, None, O.SUM, O.FP16)
             assert bits_equal(got_static, want) == 0
 

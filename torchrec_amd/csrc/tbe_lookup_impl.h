@@ -595,55 +595,6 @@ __device__ __forceinline__ void finish_bag(float (&acc)[NE], const LookupArgs& a
   store_outputs<NE>(a, pos, acc);
 }
 
-// Static mapping: lane group g of wave w of tile t owns bag (t*waves + w)*gpw + g.
-// Used for small problems, where there are not enough bags to balance.
-template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U>
-__global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupArgs a) {
-  constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;  // columns per lane
-  TRA_STAMP(0);
-  int f, lpr, tile, ci;
-  if (!locate_tile(a, f, lpr, tile, &ci)) return;
-  const FeatureDesc d = a.descs[f];
-  const int lane = threadIdx.x & (kWaveSize - 1);
-  const int wave = threadIdx.x / kWaveSize;
-  const int gpw = kWaveSize / lpr;  // lane groups (bags) per wave
-  const int g = lane / lpr;
-  const int c = lane - g * lpr;
-  const int bag_in_feat = (tile * kWavesPerBlock + wave) * gpw + g;
-  const bool active = g < gpw && bag_in_feat < a.B;
-
-  int64_t start = 0, end = 0;
-  if (active) {
-    const int64_t bag = (int64_t)d.feature * a.B + bag_in_feat;
-    start = load_index<IdxT>(a.offsets, bag);
-    end = load_index<IdxT>(a.offsets, bag + 1);
-  }
-  const int len = (int)(end - start);
-  const int max_len = wave_max(len);
-  TRA_STAMP(1);
-
-  RowWalk w;
-  w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
-  w.lane_base = a.weights + d.table_offset + w.chunk_off;
-  w.set_rows(d.rows, d.row_bytes);
-  w.count_errors = c == 0 && d.payload_off == 0;
-  w.set_position_weights(a, ci, start);
-
-  float acc[NE];
-#pragma unroll
-  for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
-  pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
-  TRA_STAMP(2);
-#ifdef TRA_INSTRUMENT
-  if ((threadIdx.x & 63) == 0)
-    a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64) * 8 + 4] = max_len;
-#endif
-  if (!active) return;
-  finish_bag<NE>(acc, a, len,
-                 (int64_t)bag_in_feat * a.out_stride + d.out_col + (int64_t)c * NE);
-  TRA_STAMP(3);
-}
-
 // Balanced mapping.  One 1024-thread block per compute unit owns a window of
 // consecutive bags (of one sub-class, possibly spanning features).  It ranks
 // them by length in LDS, longest first, and cuts the order into rounds of gpw
@@ -653,9 +604,15 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
 // w, w+4, w+8, w+12 share SIMD w & 3), which evens out the work per SIMD.  A
 // bag is still pooled whole and in id order by one lane group; there is no
 // scratch memory, atomic or pre-pass.
-constexpr int kCuThreads = 1024;
+#ifndef TRA_CU_THREADS  // (measurement builds override these two)
+#define TRA_CU_THREADS 1024
+#endif
+#ifndef TRA_MAX_WINDOW
+#define TRA_MAX_WINDOW 2048
+#endif
+constexpr int kCuThreads = TRA_CU_THREADS;
 constexpr int kCuWaves = kCuThreads / kWaveSize;
-constexpr int kMaxWindow = 2048;
+constexpr int kMaxWindow = TRA_MAX_WINDOW;
 constexpr int kBagBits = 20;  // window entry = (feature index in sub-class << 20) | sample
 
 constexpr int kLenBins = 256;
@@ -789,6 +746,104 @@ __device__ __forceinline__ void lds_barrier() {
 __device__ __forceinline__ int feat_key_pos(const LookupArgs& a, const SubClass& sc, int fi) {
   return sc.first + fi < kMaxPos ? (int)a.feat_pos[sc.first + fi]
                                  : a.descs[a.feats[sc.first + fi]].feature;
+}
+
+// Static mapping: lane group g of wave w of tile t owns bag (t*waves + w)*gpw + g.
+// Used for small problems, where there are not enough bags to balance.
+// FROM_LENGTHS: a.offsets points at the KJT's lengths; the block sums what
+// lies in front of its first bag (every block reads that prefix again: this
+// form is for calls with few bags, where a scan kernel of its own would cost
+// more than the lookup) and scans its own bags, which are consecutive.
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, bool FROM_LENGTHS = false>
+__global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupArgs a) {
+  constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;  // columns per lane
+  TRA_STAMP(0);
+  int f, lpr, tile, ci;
+  if (!locate_tile(a, f, lpr, tile, &ci)) return;
+  const FeatureDesc d = a.descs[f];
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int wave = threadIdx.x / kWaveSize;
+  const int gpw = kWaveSize / lpr;  // lane groups (bags) per wave
+  const int g = lane / lpr;
+  const int c = lane - g * lpr;
+  const int bag_in_feat = (tile * kWavesPerBlock + wave) * gpw + g;
+  const bool active = g < gpw && bag_in_feat < a.B;
+
+  int64_t start = 0;
+  int len = 0;
+  if (FROM_LENGTHS) {
+    using Sum = typename SumOf<IdxT>::type;
+    constexpr int V = 16 / (int)sizeof(IdxT);
+    struct __align__(16) Vec { IdxT v[V]; };
+    __shared__ Sum s_front[kWavesPerBlock];
+    __shared__ Sum s_wave_tot[kWavesPerBlock];
+    const IdxT* lengths = reinterpret_cast<const IdxT*>(a.offsets);
+    // this lane group's own length first: its load shares the latency of the prefix loads
+    const int64_t bag = (int64_t)d.feature * a.B + min(bag_in_feat, a.B - 1);
+    const Sum raw = active ? (Sum)lengths[bag] : (Sum)0;
+    // sum(lengths[0 .. p)), p = position of the block's first bag (16-byte steps, then the rest)
+    const int64_t p = (int64_t)d.feature * a.B + (int64_t)tile * kWavesPerBlock * gpw;
+    const int nvec = (int)(p / V);
+    Sum part = 0;
+    for (int v0 = 0; v0 < nvec; v0 += 4 * kBlockThreads) {
+      Vec x[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) x[k] = reinterpret_cast<const Vec*>(lengths)[min(v0 + k * kBlockThreads + (int)threadIdx.x, nvec - 1)];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        Sum sum = 0;
+#pragma unroll
+        for (int i = 0; i < V; ++i) sum += (Sum)x[k].v[i];
+        part += v0 + k * kBlockThreads + (int)threadIdx.x < nvec ? sum : (Sum)0;
+      }
+    }
+    {
+      const int64_t ti = (int64_t)nvec * V + threadIdx.x;
+      if (ti < p) part += (Sum)lengths[ti];
+    }
+    // bag starts inside the block: scan over the lane groups (the group's first
+    // lane carries its length), then over the block's waves
+    const Sum incl = wave_scan_incl(c == 0 && g < gpw ? raw : (Sum)0);
+    const Sum front_w = wave_last(wave_scan_incl(part));
+    if (lane == kWaveSize - 1) s_wave_tot[wave] = incl;
+    if (lane == 0) s_front[wave] = front_w;
+    __syncthreads();
+    Sum before = 0, front = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      front += s_front[w];
+      if (w < wave) before += s_wave_tot[w];
+    }
+    start = (int64_t)(front + before + incl - raw);
+    len = raw > 0 ? (int)raw : 0;
+  } else if (active) {
+    const int64_t bag = (int64_t)d.feature * a.B + bag_in_feat;
+    start = load_index<IdxT>(a.offsets, bag);
+    len = (int)(load_index<IdxT>(a.offsets, bag + 1) - start);
+  }
+  const int max_len = wave_max(len);
+  TRA_STAMP(1);
+
+  RowWalk w;
+  w.chunk_off = Traits<DTYPE>::kHeader + d.payload_off + c * CB;
+  w.lane_base = a.weights + d.table_offset + w.chunk_off;
+  w.set_rows(d.rows, d.row_bytes);
+  w.count_errors = c == 0 && d.payload_off == 0;
+  w.set_position_weights(a, ci, start);
+
+  float acc[NE];
+#pragma unroll
+  for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
+  pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+  TRA_STAMP(2);
+#ifdef TRA_INSTRUMENT
+  if ((threadIdx.x & 63) == 0)
+    a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64) * 8 + 4] = max_len;
+#endif
+  if (!active) return;
+  finish_bag<NE>(acc, a, len,
+                 (int64_t)bag_in_feat * a.out_stride + d.out_col + (int64_t)c * NE);
+  TRA_STAMP(3);
 }
 
 // FROM_LENGTHS: a.offsets points at the KJT's lengths instead of its offsets
@@ -993,7 +1048,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   // measured the same: the waves that finish early leave the CU's memory
   // pipeline to the ones still running.)
   for (int pass = 0; pass * kCuWaves < rounds; ++pass) {
-    const int slot = pass * 4 + (wave >> 2);
+    const int slot = pass * (kCuWaves / 4) + (wave >> 2);
     const int r = slot * 4 + ((slot & 1) ? 3 - (wave & 3) : (wave & 3));
     if (r >= rounds) continue;
     const int pos = r * gpw + g;
@@ -1126,6 +1181,9 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
     else if (p.balanced)                                                                       \
       hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kCuThreads),   \
                          p.lds_bytes, stream, a);                                              \
+    else if (p.from_lengths)                                                                   \
+      hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, 4, true>), g,                  \
+                         dim3(kBlockThreads), 0, stream, a);                                   \
     else                                                                                       \
       hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kBlockThreads), 0, \
                          stream, a);                                                           \

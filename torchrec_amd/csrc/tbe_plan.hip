@@ -450,6 +450,20 @@ static bool fused_scan_possible(const tra_tbe* tbe, int32_t batch_size, int32_t 
   return (int64_t)tbe->classes.size() * (13 + n / 4000) < 70;
 }
 
+// A pooled call too small for the window kernel whose lengths are few enough
+// that every block of the static kernel can sum the ones in front of its bags
+// itself: one launch instead of a scan and a lookup.
+constexpr int64_t kSmallFusedMaxLengths = 16384;
+
+static bool small_fused_scan_possible(const tra_tbe* tbe, int32_t batch_size, int32_t num_keys,
+                                      int64_t num_indices, int32_t pooling_mode, const void* lengths) {
+  if (pooling_mode == TRA_POOL_NONE || batch_size <= 0 || tbe->num_features == 0) return false;
+  if ((uintptr_t)lengths % 16 != 0 || g_ovr.fused_scan == 0) return false;
+  const Tuning tune = choose_tuning(tbe->num_cus, (int64_t)tbe->num_features * batch_size, num_indices);
+  if (use_window_kernel(tbe, tune, false, batch_size)) return false;
+  return (int64_t)num_keys * batch_size <= kSmallFusedMaxLengths;
+}
+
 int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
                         int32_t pooling_mode, int32_t lengths_num_keys, char* buf,
                         int32_t buf_len) {
@@ -462,8 +476,10 @@ int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
   const bool balanced = use_window_kernel(tbe, tune, nobag, batch_size);
   // lengths entry point: same decision as tra_tbe_forward_lengths (aligned lengths assumed)
   const bool fused = lengths_num_keys > 0 &&
-                     fused_scan_possible(tbe, batch_size, lengths_num_keys, num_indices, pooling_mode,
-                                         (const void*)16);
+                     (fused_scan_possible(tbe, batch_size, lengths_num_keys, num_indices, pooling_mode,
+                                          (const void*)16) ||
+                      small_fused_scan_possible(tbe, batch_size, lengths_num_keys, num_indices, pooling_mode,
+                                                (const void*)16));
   static const char* const kDtypeName[] = {"fp32", "fp16", "int8", "int4", "int2"};
   std::string text;
   for (const LaunchClass& cls : tbe->classes) {
@@ -784,7 +800,8 @@ static int forward_lengths_impl(tra_tbe_t tbe, const void* weights, const void* 
     set_error("tra_tbe_forward_lengths: null lengths");
     return TRA_ERR_INVALID_ARGUMENT;
   }
-  if (fused_scan_possible(tbe, batch_size, num_keys, num_indices, pooling_mode, lengths))
+  if (fused_scan_possible(tbe, batch_size, num_keys, num_indices, pooling_mode, lengths) ||
+      small_fused_scan_possible(tbe, batch_size, num_keys, num_indices, pooling_mode, lengths))
     return forward_impl(tbe, weights, indices, lengths, true, idx_is_i64, per_sample_weights,
                         batch_size, num_indices, pooling_mode, out_dtype, out, out_stride, stream, pw);
   // Offsets first, then the ordinary lookup.

@@ -28,6 +28,12 @@ from torch import nn, Tensor
 from torchrec_amd import _lib
 from torchrec_amd.tbe.enums import BoundsCheckMode, EmbeddingLocation, PoolingMode, SparseType
 
+# TORCHREC_AMD_BOUNDS_CHECK=1 (read when this module is imported): every forward
+# fetches the count of out-of-range ids and raises if there were any (synchronizes).
+_ENV_BOUNDS_CHECK = os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1"
+_INT_DTYPES = (torch.int32, torch.int64)
+_BOUNDS_FATAL = int(BoundsCheckMode.FATAL)
+
 _SUPPORTED_WEIGHTS = (SparseType.FP32, SparseType.FP16, SparseType.INT8, SparseType.INT4, SparseType.INT2)
 _TABLE_ALIGNMENT = 256
 
@@ -142,6 +148,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self._identity_positions: Tuple[int, ...] = tuple(range(len(self.feature_table_map)))
         self._num_keys: Dict[Tuple[int, ...], int] = {}
         self._workspace: Dict[int, Tensor] = {}  # per stream: scratch of forward(offsets=None, lengths=...)
+        self._ws_bytes: Dict[Tuple[int, int, int], int] = {}  # size of that scratch per (keys, batch size, id width)
         self._weights_initialized = False
         self.weight_initialized = False
         self.register_buffer("weights_dev", torch.empty(0, dtype=torch.uint8, device=device), persistent=False)
@@ -326,21 +333,28 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             raise _lib.TorchrecAmdError("weights are not initialized (call initialize_weights())")
         if self.weights_dev.device != dev:  # e.g. the buffer was replaced by hand
             raise _lib.TorchrecAmdError(f"packed weights are on {self.weights_dev.device}, the operator on {dev}")
-        _lib.require_gpu(indices, "indices")
-        if indices.dtype not in (torch.int32, torch.int64):
-            raise TypeError(f"indices must be int32 or int64, got {indices.dtype}")
-        indices = indices.contiguous()
+        idt = indices.dtype
+        if not indices.is_cuda:
+            _lib.require_gpu(indices, "indices")
+        if idt not in _INT_DTYPES:
+            raise TypeError(f"indices must be int32 or int64, got {idt}")
+        if not indices.is_contiguous():
+            indices = indices.contiguous()
         if offsets is None:
             assert lengths is not None and batch_size is not None, "offsets=None needs lengths and batch_size"
-            _lib.require_gpu(lengths, "lengths")
-            if lengths.dtype != indices.dtype:
-                lengths = lengths.to(indices.dtype)
-            lengths = lengths.contiguous().view(-1)
+            if not lengths.is_cuda:
+                _lib.require_gpu(lengths, "lengths")
+            if lengths.dtype != idt:
+                lengths = lengths.to(idt)
+            if lengths.dim() != 1 or not lengths.is_contiguous():
+                lengths = lengths.contiguous().view(-1)
         else:
-            _lib.require_gpu(offsets, "offsets")
-            if offsets.dtype != indices.dtype:
-                offsets = offsets.to(indices.dtype)
-            offsets = offsets.contiguous()
+            if not offsets.is_cuda:
+                _lib.require_gpu(offsets, "offsets")
+            if offsets.dtype != idt:
+                offsets = offsets.to(idt)
+            if not offsets.is_contiguous():
+                offsets = offsets.contiguous()
         F = len(self.feature_table_map)
         positions: Optional[Tuple[int, ...]] = None
         if feature_positions is not None:
@@ -394,7 +408,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 assert out.shape[0] >= B and out.shape[1] >= out_col + self.total_D
         out_stride = out.stride(0)
         out_ptr = out.data_ptr() + out_col * out.element_size()
-        i64 = int(indices.dtype == torch.int64)
+        i64 = int(idt == torch.int64)
         if pos_args is not None:
             table, c_start, c_len, n_k = pos_args
             stream = _lib.current_stream(dev)
@@ -415,7 +429,10 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 )
             )
         elif offsets is None:
-            ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
+            ws_key = (k_total, B, i64)
+            ws_bytes = self._ws_bytes.get(ws_key)
+            if ws_bytes is None:
+                ws_bytes = self._ws_bytes[ws_key] = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
             stream = _lib.current_stream(dev)
             # one scratch buffer per stream: calls queued on different streams must not share it
             ws = self._workspace.get(stream)
@@ -436,7 +453,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                     self.output_dtype, out_ptr, out_stride, _lib.current_stream(dev),
                 )
             )
-        if self.bounds_check_mode_int == int(BoundsCheckMode.FATAL) or os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1":
+        if _ENV_BOUNDS_CHECK or self.bounds_check_mode_int == _BOUNDS_FATAL:
             bad = self.out_of_range_count()
             if bad:
                 raise IndexError(f"{bad} embedding indices were out of range")
