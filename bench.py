@@ -637,11 +637,21 @@ def main():
     torch.cuda.synchronize()
     del cal
 
+    # HBM traffic per launch is not measured in this run: it comes from the stored
+    # hardware-counter profile of the same workload, named here with the commit
+    # whose kernels that profile measured (a kernel changed since then makes it stale).
     traffic = None
+    traffic_source = None
     tpath = os.path.join(ROOT, "profiles", f"{args.config}_lookup_traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+            stored = json.load(open(tpath))
+            traffic = stored.get("hbm_bytes_per_launch")
+            traffic_source = {
+                "file": os.path.relpath(tpath, ROOT),
+                "measured_at_commit": stored.get("measured_at_commit"),
+                "note": "from the stored rocprofv3 counter runs (FETCH_SIZE, WRITE_SIZE x copy-kernel calibration), not measured in this run",
+            }
         except Exception:
             traffic = None
 
@@ -673,6 +683,7 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
+            "traffic_source": traffic_source,
             "kernel": launches[0].split(" ")[0],
             "launches_per_call": launches,
             "kernel_ms": kernel_ms,
