@@ -35,12 +35,15 @@ struct SubClass {
   int32_t tiles_per_feat;  // blocks per feature
   int32_t tile_start;      // first block of this sub-class in the grid
   int32_t window;          // window kernel: bags per block
+  int32_t key0;            // key position of the first feature when the sub-class's features sit
+                           // at consecutive key positions (feature fi at key0 + fi), else -1
 };
 
 struct LookupArgs {
   const uint8_t* weights;
   const FeatureDesc* descs;  // all features of the plan (device)
   const int32_t* feats;      // feature ids of this launch (device)
+  const FeatureDesc* cdescs; // the same features' descriptors in launch order: cdescs[i] == descs[feats[i]]
   const void* indices;
   const void* offsets;
   const float* psw;
@@ -744,6 +747,7 @@ __device__ __forceinline__ void lds_barrier() {
 // Position of feature `fi` of a sub-class among the input keys: from the launch
 // arguments when the class is small enough, else from the descriptors.
 __device__ __forceinline__ int feat_key_pos(const LookupArgs& a, const SubClass& sc, int fi) {
+  if (sc.key0 >= 0) return sc.key0 + fi;  // no load: the bag bounds can be requested at once
   return sc.first + fi < kMaxPos ? (int)a.feat_pos[sc.first + fi]
                                  : a.descs[a.feats[sc.first + fi]].feature;
 }
@@ -900,7 +904,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   // round does not start with two dependent global loads.
   {
     const int nfeat = min((q0 + nb - 1) / a.B - fi_lo + 1, kMaxWinFeat);
-    if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = a.descs[a.feats[sc.first + fi_lo + threadIdx.x]];
+    if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = a.cdescs[sc.first + fi_lo + threadIdx.x];
   }
   // From lengths: the total of everything in front of the window.  Its loads
   // go out after the window's own (loads return in order: whatever is waited
@@ -971,7 +975,8 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     // key position follows directly, the run simply continues.
     const int fi_hi = (q0 + nb - 1) / a.B;
     bool one_run = true;
-    for (int fi = fi_lo; fi < fi_hi; ++fi) one_run = one_run && feat_key_pos(a, sc, fi + 1) == feat_key_pos(a, sc, fi) + 1;
+    if (sc.key0 < 0)
+      for (int fi = fi_lo; fi < fi_hi; ++fi) one_run = one_run && feat_key_pos(a, sc, fi + 1) == feat_key_pos(a, sc, fi) + 1;
     if (one_run) {
       if (2 * t < nb) s_start[2 * t] = (int64_t)(front + excl);
       if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(front + excl + x0);
@@ -1057,7 +1062,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     const uint32_t ent = s_ent[i];
     const int fi = (int)(ent >> kBagBits);
     const int b = (int)(ent & ((1u << kBagBits) - 1));
-    const FeatureDesc d = fi - fi_lo < kMaxWinFeat ? s_desc[fi - fi_lo] : a.descs[a.feats[sc.first + fi]];
+    const FeatureDesc d = fi - fi_lo < kMaxWinFeat ? s_desc[fi - fi_lo] : a.cdescs[sc.first + fi];
     const int64_t start = s_start[i];
     const int len = active ? max(s_len[i], 0) : 0;
     // The round's trip count.  Lengths below 192 have a sort bin each, so

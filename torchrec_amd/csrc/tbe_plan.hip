@@ -176,6 +176,7 @@ struct tra_tbe {
   std::vector<FeatureDesc> slices;  // host copy
   FeatureDesc* slices_dev = nullptr;
   int32_t* feats_dev = nullptr;  // all classes' slice lists, concatenated
+  FeatureDesc* cdescs_dev = nullptr;  // the descriptors in that order: cdescs[i] = slices[feats[i]]
   unsigned long long* err_dev = nullptr;
   void* static_scratch = nullptr;  // this device's copy of the library's static scratch array
   std::vector<LaunchClass> classes;
@@ -383,6 +384,12 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
       e = hipMemcpy(plan->feats_dev, all_feats.data(), total * sizeof(int32_t),
                     hipMemcpyHostToDevice);
     }
+    if (e == hipSuccess) e = hipMalloc((void**)&plan->cdescs_dev, total * sizeof(FeatureDesc));
+    if (e == hipSuccess) {
+      std::vector<FeatureDesc> ordered;
+      for (int32_t id : all_feats) ordered.push_back(plan->slices[id]);
+      e = hipMemcpy(plan->cdescs_dev, ordered.data(), total * sizeof(FeatureDesc), hipMemcpyHostToDevice);
+    }
   }
   if (e == hipSuccess) e = hipMalloc((void**)&plan->err_dev, sizeof(unsigned long long));
   if (e == hipSuccess) e = hipMemset(plan->err_dev, 0, sizeof(unsigned long long));
@@ -401,6 +408,7 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     memset(&a, 0, sizeof(a));
     a.descs = plan->slices_dev;
     a.feats = cls.feats_dev;
+    a.cdescs = plan->cdescs_dev + (cls.feats_dev - plan->feats_dev);
     a.err_count = plan->err_dev;
     for (size_t i = 0; i < cls.feats.size() && i < (size_t)kMaxPos; ++i)
       a.feat_pos[i] = (int16_t)plan->slices[cls.feats[i]].feature;
@@ -414,6 +422,7 @@ int tra_tbe_destroy(tra_tbe_t tbe) {
   if (!tbe) return TRA_OK;
   if (tbe->slices_dev) (void)hipFree(tbe->slices_dev);
   if (tbe->feats_dev) (void)hipFree(tbe->feats_dev);
+  if (tbe->cdescs_dev) (void)hipFree(tbe->cdescs_dev);
   if (tbe->err_dev) (void)hipFree(tbe->err_dev);
   delete tbe;
   return TRA_OK;
@@ -561,6 +570,9 @@ static void compute_geometry(const tra_tbe* tbe, const Tuning& tune, bool balanc
       sc.first = (int)i;
       sc.count = (int)(j - i);
       sc.lpr = cls.lprs[i];
+      sc.key0 = tbe->slices[cls.feats[i]].feature;
+      for (size_t k = i; k < j; ++k)
+        if (tbe->slices[cls.feats[k]].feature != sc.key0 + (int)(k - i)) sc.key0 = -1;
       const int gpw = kWaveSize / sc.lpr;
       const int per_block = kWavesPerBlock * gpw;
       sc.tile_start = grid;
