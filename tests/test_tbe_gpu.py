@@ -88,7 +88,8 @@ def test_mixed_group_one_call():
 
 @pytest.mark.parametrize("dtype,dim", [(O.INT8, 8), (O.INT8, 12), (O.INT8, 24), (O.INT4, 8), (O.INT4, 24),
                                        (O.INT4, 40), (O.INT2, 16), (O.INT2, 48), (O.FP16, 2), (O.FP16, 6),
-                                       (O.FP16, 20), (O.FP32, 1), (O.FP32, 3), (O.FP32, 10), (O.INT8, 1040),
+                                       (O.FP16, 20), (O.FP32, 1), (O.FP32, 3), (O.FP32, 10), (O.INT8, 1040), (O.INT8, 520), (O.INT4, 1048),
+                                       (O.INT2, 2064),
                                        (O.FP16, 1000), (O.FP32, 520)])
 def test_odd_dims(dtype, dim):
     """Payloads that are not multiples of 16 bytes (8- and 4-byte lane chunks) and
@@ -100,6 +101,30 @@ def test_odd_dims(dtype, dim):
         lengths, offsets, ids = make_bags(rng, [rows], B, 9)
         got, want = run_both(tbe, store, [0], B, ids, offsets, None, pooling, O.FP32)
         assert bits_equal(got, want) == 0
+
+
+@pytest.mark.parametrize("route", ["static", "window", "lengths", "static-lengths"])
+def test_wide_rows_next_to_ordinary_ones(tuning, route):
+    """int-N rows too wide for one wave of 8- or 4-byte lane chunks are cut into column slices and get
+    a launch class of their own (the header is loaded separately there); ordinary rows of the same
+    weight type keep the class whose first lane receives the header with its chunk.  Both in one
+    operator, weighted MEAN, every pooled kernel and both entries, against the oracle."""
+    tuning(balanced=1 if route in ("window", "lengths") else 0)
+    rng = np.random.default_rng(len(route))
+    rows, B = 400, 160
+    specs = [(O.INT8, rows, 520), (O.INT4, rows, 128), (O.INT8, rows, 64), (O.INT4, rows, 1048), (O.INT2, rows, 2064),
+             (O.INT2, rows, 64)]
+    ftm = [0, 1, 2, 3, 4, 5, 1]
+    tbe, store = build(rng, specs, ftm, O.MEAN, O.FP16, 16)
+    lengths, offsets, ids = make_bags(rng, [rows] * len(ftm), B, 30)
+    psw = rng.uniform(-1, 1, len(ids)).astype(np.float32)
+    want = O.tbe_forward(store, ftm, B, ids, offsets, psw, O.MEAN, O.FP16)
+    if route.endswith("lengths"):
+        got = _from_lengths(tbe, ids, lengths, psw, B)
+    else:
+        got = tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV), torch.from_numpy(psw).to(DEV)).cpu().numpy()
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == 0
 
 
 def test_edge_bags():

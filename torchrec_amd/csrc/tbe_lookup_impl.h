@@ -90,6 +90,25 @@ struct Traits<TRA_INT2> {
   static constexpr int kBits = 2;
   static constexpr int kHeader = 4;
 };
+// Kernel-internal type codes for int-N rows too wide for one wave of lanes
+// (more than 64 chunks of at most 8 bytes): such a row is cut into column
+// slices, and only its first slice has the row header in front of it, so
+// these variants load the header on its own (kHeaderWithChunk false).
+constexpr int kSplitHeader = 16;
+template <>
+struct Traits<TRA_INT8 + kSplitHeader> : Traits<TRA_INT8> {};
+template <>
+struct Traits<TRA_INT4 + kSplitHeader> : Traits<TRA_INT4> {};
+template <>
+struct Traits<TRA_INT2 + kSplitHeader> : Traits<TRA_INT2> {};
+// The weight type proper of a kernel type code.
+constexpr int base_type(int dtype) { return dtype >= kSplitHeader ? dtype - kSplitHeader : dtype; }
+// Does a lane load the dword in front of its chunk together with the chunk
+// (for a row's first lane: the header)?  Rows with a header, 8- or 4-byte
+// chunks, whole row in one slice.
+template <int DTYPE, int CB>
+constexpr bool header_with_chunk() { return Traits<DTYPE>::kHeader != 0 && CB <= 8 && DTYPE < kSplitHeader; }
+
 template <>
 struct Traits<TRA_FP16> {
   static constexpr int kBits = 16;
@@ -150,9 +169,10 @@ __device__ __forceinline__ void fma_step(float& acc, float s, float q, float b) 
 // number, so the fused multiply-add rounds identically.  With per-sample
 // weights the scale w*scale may be subnormal, where that division is inexact,
 // so the fields are shifted down instead.
-template <int DTYPE, bool WEIGHTED>
+template <int DTYPE_CODE, bool WEIGHTED>
 __device__ __forceinline__ void accumulate_dword(float* acc, uint32_t x, float s,
                                                  float b) {
+  constexpr int DTYPE = base_type(DTYPE_CODE);
   if constexpr (DTYPE == TRA_INT8) {
     fma_step(acc[0], s, byte_to_float<0>(x), b);
     fma_step(acc[1], s, byte_to_float<1>(x), b);
@@ -246,6 +266,9 @@ struct RowWalk {
   uint32_t row_bytes;
   int chunk_off;
   bool count_errors;
+  // Where a lane loads the dword in front of its chunk together with the chunk
+  // (header_with_chunk), the row's header arrives in the row's first lane.
+  int hdr_lane;
   // position weighting: this bag's weight vector (always readable), its last
   // index, whether the feature has one at all, and where the bag starts
   const float* pw;
@@ -316,11 +339,20 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
     const int64_t idc = valid ? (int64_t)id : 0;
     chunk = lane_base + idc * (int64_t)w.row_bytes;
   }
-  if constexpr (Traits<DTYPE>::kHeader != 0)
-    r.hdr = *reinterpret_cast<const uint32_t*>(chunk - chunk_off);
-  else
-    r.hdr = 0;
-  r.d = load_chunk<CB>(chunk);
+  if constexpr (header_with_chunk<DTYPE, CB>()) {
+    // One load: the dword in front of the lane's chunk and the chunk.  For the
+    // row's first lane that dword is the header; consume_row hands it round.
+    const Chunk<CB + 4> t = load_chunk<CB + 4>(chunk - 4);
+    r.hdr = t.v[0];
+#pragma unroll
+    for (int i = 0; i < CB / 4; ++i) r.d.v[i] = t.v[i + 1];
+  } else {
+    if constexpr (Traits<DTYPE>::kHeader != 0)
+      r.hdr = *reinterpret_cast<const uint32_t*>(chunk - chunk_off);
+    else
+      r.hdr = 0;
+    r.d = load_chunk<CB>(chunk);
+  }
   if constexpr (WEIGHTED) {
     using UIdxT = typename std::make_unsigned<IdxT>::type;
     if constexpr (WEIGHTED == kByPosition) {
@@ -348,8 +380,11 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
 // q is a finite integer.  For fp16 / fp32 rows the payload of an invalid row is
 // zeroed as well, so a stored inf / nan in row 0 cannot leak in.
 template <int DTYPE, int CB, bool WEIGHTED>
-__device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r) {
+__device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r0, const RowWalk& w) {
   constexpr int EPD = 32 / Traits<DTYPE>::kBits;  // elements per dword
+  RowBuf<CB> r = r0;
+  if constexpr (header_with_chunk<DTYPE, CB>())
+    r.hdr = (uint32_t)__shfl((int)r0.hdr, w.hdr_lane, kWaveSize);  // the header sits with the row's first lane
   float s, b;
   if constexpr (Traits<DTYPE>::kHeader != 0) {
     if constexpr (WEIGHTED) {
@@ -494,7 +529,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], idB[u], start + it + U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u]);
+      if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u], w);
     if (it + U >= max_len) break;
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -504,7 +539,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], idA[u], start + it + 2 * U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u]);
+      if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u], w);
   }
   // Bad ids are counted by the lane that owns column 0.
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
@@ -574,7 +609,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u]);
+      if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u], w);
     if (it + U >= max_len) break;
     if constexpr (TWO_BATCHES) advance(); else enter(it + 2 * U);
 #pragma unroll
@@ -582,7 +617,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
       bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u]);
+      if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u], w);
   }
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
 }
@@ -887,6 +922,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
   w.lane_base = a.weights + d.table_offset + w.chunk_off;
   w.set_rows(d.rows, d.row_bytes);
   w.count_errors = c == 0 && d.payload_off == 0;
+  w.hdr_lane = lane - c;
   w.set_position_weights(a, ci, start);
 
   float acc[NE];
@@ -1129,6 +1165,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     w.lane_base = a.weights + d.table_offset + w.chunk_off;
     w.set_rows(d.rows, d.row_bytes);
     w.count_errors = c == 0 && d.payload_off == 0;
+    w.hdr_lane = lane - c;
     w.set_position_weights(a, sc.first + fi, start);
 
     float acc[NE];
@@ -1181,6 +1218,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
   w.lane_base = a.weights + d.table_offset + w.chunk_off;
   w.set_rows(d.rows, d.row_bytes);
   w.count_errors = c == 0 && d.payload_off == 0;
+  w.hdr_lane = lane - c;
   for (int64_t j = first + (int64_t)tile * rows_per_block + wave * gpw + g; j < last;
        j += stride) {
     RowBuf<CB> r;
@@ -1190,7 +1228,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
     float acc[NE];
 #pragma unroll
     for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
-    consume_row<DTYPE, CB, false>(acc, r);
+    consume_row<DTYPE, CB, false>(acc, r, w);
     store_outputs<NE>(a, j * (int64_t)d.dim + d.payload_off * 8 / Traits<DTYPE>::kBits + (int64_t)c * NE,
                       acc);
   }
@@ -1200,6 +1238,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
 struct LaunchClass {
   int dtype;
   int cb;
+  bool split = false;  // rows cut into several column slices, header loaded on its own (kSplitHeader)
   std::vector<int32_t> feats;  // plan order: sorted by lpr
   std::vector<int32_t> lprs;   // lanes per row of each feature
   int32_t* feats_dev = nullptr;
@@ -1244,7 +1283,9 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
       hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kBlockThreads), 0, \
                          stream, a);                                                           \
   } while (0)
-  if (a.posw != nullptr) {
+  if constexpr (DTYPE >= kSplitHeader) {  // (one unroll depth for the rare split rows)
+    if (a.posw != nullptr) TRA_POOLED(kByPosition, 4); else if (p.weighted) TRA_POOLED(kPerSample, 4); else TRA_POOLED(kUnweighted, 4);
+  } else if (a.posw != nullptr) {
     TRA_POOLED(kByPosition, 4);  // (one unroll depth: the others are tuning variants)
   } else if (p.weighted) {
     if (p.unroll >= 8) TRA_POOLED(kPerSample, 8); else if (p.unroll >= 4) TRA_POOLED(kPerSample, 4); else TRA_POOLED(kPerSample, 2);
@@ -1270,7 +1311,9 @@ int launch_lookup_cb(const LookupArgs& a, const LaunchParams& p, hipStream_t str
   int launch_lookup<DTYPE>(const LookupArgs& a, int cb, const LaunchParams& p,            \
                            hipStream_t stream) {                                          \
     switch (cb) {                                                                         \
-      case 16: return launch_lookup_cb<DTYPE, 16>(a, p, stream);                          \
+      case 16:                                                                            \
+        if constexpr (DTYPE < kSplitHeader) return launch_lookup_cb<DTYPE, 16>(a, p, stream); \
+        break;                                                                            \
       case 8: return launch_lookup_cb<DTYPE, 8>(a, p, stream);                            \
       case 4: return launch_lookup_cb<DTYPE, 4>(a, p, stream);                            \
     }                                                                                     \

@@ -3,4 +3,5 @@
 
 namespace tra {
 TRA_DEFINE_LAUNCH(TRA_INT2)
+TRA_DEFINE_LAUNCH(TRA_INT2 + kSplitHeader)
 }  // namespace tra

@@ -3,4 +3,5 @@
 
 namespace tra {
 TRA_DEFINE_LAUNCH(TRA_INT4)
+TRA_DEFINE_LAUNCH(TRA_INT4 + kSplitHeader)
 }  // namespace tra

@@ -3,4 +3,5 @@
 
 namespace tra {
 TRA_DEFINE_LAUNCH(TRA_INT8)
+TRA_DEFINE_LAUNCH(TRA_INT8 + kSplitHeader)
 }  // namespace tra

@@ -6,6 +6,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <tuple>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -35,6 +36,12 @@ template <>
 int launch_lookup<TRA_INT4>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
 int launch_lookup<TRA_INT2>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
+template <>
+int launch_lookup<TRA_INT8 + kSplitHeader>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
+template <>
+int launch_lookup<TRA_INT4 + kSplitHeader>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
+template <>
+int launch_lookup<TRA_INT2 + kSplitHeader>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
 int launch_lookup<TRA_FP16>(const LookupArgs&, int, const LaunchParams&, hipStream_t);
 template <>
@@ -268,7 +275,8 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
   auto plan = new tra_tbe();
   plan->num_features = num_features;
   int col = 0;
-  std::map<std::pair<int, int>, std::vector<int>> by_class;  // (dtype, cb) -> slice ids
+  // (dtype, cb, rows cut into several slices) -> slice ids
+  std::map<std::tuple<int, int, int>, std::vector<int>> by_class;
   std::vector<int> slice_lpr;
   for (int f = 0; f < num_features; ++f) {
     const int t = feature_table_map[f];
@@ -293,6 +301,10 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
       if ((force == 8 || force == 4) && force < cb && payload % force == 0) cb = force;
     }
     const int max_slice = cb * kWaveSize;  // bytes one wave-wide lane group covers
+    // A row with a header whose lanes take 8 or 4 bytes normally gets its header with the
+    // first lane's chunk; cut into several slices, only the first slice could, so all its
+    // slices go to a launch class of their own that loads the header separately.
+    const int split = payload > max_slice && header_bytes(s.dtype) != 0 && cb <= 8 ? 1 : 0;
     for (int off = 0; off < payload; off += max_slice) {
       const int bytes = std::min(max_slice, payload - off);
       FeatureDesc d;
@@ -304,7 +316,7 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
       d.dtype = s.dtype;
       d.feature = feature_positions ? feature_positions[f] : f;
       d.payload_off = off;
-      by_class[{s.dtype, cb}].push_back((int)plan->slices.size());
+      by_class[{s.dtype, cb, split}].push_back((int)plan->slices.size());
       plan->slices.push_back(d);
       slice_lpr.push_back(bytes / cb);
     }
@@ -330,8 +342,9 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
         ++distinct;
         last_lpr = slice_lpr[id];
       }
-      cur.dtype = kv.first.first;
-      cur.cb = kv.first.second;
+      cur.dtype = std::get<0>(kv.first);
+      cur.cb = std::get<1>(kv.first);
+      cur.split = std::get<2>(kv.first) != 0;
       cur.feats.push_back(id);
       cur.lprs.push_back(slice_lpr[id]);
     }
@@ -759,9 +772,15 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     lp.from_lengths = from_lengths;
     int rc;
     switch (cls.dtype) {
-      case TRA_INT8: rc = launch_lookup<TRA_INT8>(a, cls.cb, lp, s); break;
-      case TRA_INT4: rc = launch_lookup<TRA_INT4>(a, cls.cb, lp, s); break;
-      case TRA_INT2: rc = launch_lookup<TRA_INT2>(a, cls.cb, lp, s); break;
+      case TRA_INT8:
+        rc = cls.split ? launch_lookup<TRA_INT8 + kSplitHeader>(a, cls.cb, lp, s) : launch_lookup<TRA_INT8>(a, cls.cb, lp, s);
+        break;
+      case TRA_INT4:
+        rc = cls.split ? launch_lookup<TRA_INT4 + kSplitHeader>(a, cls.cb, lp, s) : launch_lookup<TRA_INT4>(a, cls.cb, lp, s);
+        break;
+      case TRA_INT2:
+        rc = cls.split ? launch_lookup<TRA_INT2 + kSplitHeader>(a, cls.cb, lp, s) : launch_lookup<TRA_INT2>(a, cls.cb, lp, s);
+        break;
       case TRA_FP16: rc = launch_lookup<TRA_FP16>(a, cls.cb, lp, s); break;
       default: rc = launch_lookup<TRA_FP32>(a, cls.cb, lp, s); break;
     }
