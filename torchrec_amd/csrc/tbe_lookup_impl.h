@@ -602,7 +602,28 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
 #pragma unroll
   for (int u = 0; u < U; ++u)
     bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(u), start + u, last, a, w);
-  for (int it = 0; it < max_len; it += 2 * U) {
+  int it = 0;
+  if constexpr (TWO_BATCHES) {
+    // Whole iterations (2 * U rows, all inside the longest bag) run without the
+    // per-row tests: every buffer is consumed on the way round, so the
+    // compiler knows at the top of the loop that only the newest batch and
+    // the id block are in flight and need not drain them before it reuses a
+    // consumed buffer's registers.  The last, partial iteration follows below.
+    for (; it + 2 * U <= max_len; it += 2 * U) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
+#pragma unroll
+      for (int u = 0; u < U; ++u) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u], w);
+      advance();
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
+#pragma unroll
+      for (int u = 0; u < U; ++u) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u], w);
+    }
+  }
+  for (; it < max_len; it += 2 * U) {
     if constexpr (!TWO_BATCHES) enter(it + U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
