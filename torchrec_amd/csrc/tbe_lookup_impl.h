@@ -963,7 +963,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
 // and the block derives its bags' start positions itself: one block-wide sum
 // of everything in front of the window plus a scan of the window in LDS.
 template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, bool FROM_LENGTHS = false>
-__global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupArgs a) {
+__global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const void* p_offsets, const FeatureDesc* p_cdescs, int32_t p_B, int32_t p_xcd_blocks, int32_t p_xcd_count, int32_t p_n_sub, int32_t p_window0, int32_t p_count0, int32_t p_key0, const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;
   extern __shared__ unsigned char tra_dyn_smem[];  // only its size matters (one block per CU)
   __shared__ int64_t s_start[kMaxWindow];
@@ -977,27 +977,41 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   TRA_STAMP(0);
   // Block -> (sub-class, window).  Consecutive windows go to the same XCD
   // (blocks are dealt round-robin to the 8 XCDs), so each L2 sees few tables.
+  // The leading kernel parameters repeat what the first fetches need (the
+  // hardware preloads them into SGPRs): the block's bag bounds can be
+  // requested without waiting for the launch arguments to arrive from memory.
   int blk = blockIdx.x;
-  if (a.xcd_blocks > 0) blk = (blk % a.xcd_count) * a.xcd_blocks + blk / a.xcd_count;
-  int s = 0;
+  if (p_xcd_blocks > 0) blk = (blk % p_xcd_count) * p_xcd_blocks + blk / p_xcd_count;
+  SubClass sc;
+  if (p_n_sub == 1) {
+    sc.first = 0;
+    sc.count = p_count0;
+    sc.lpr = a.sub[0].lpr;
+    sc.tiles_per_feat = 0;
+    sc.tile_start = 0;
+    sc.window = p_window0;
+    sc.key0 = p_key0;
+  } else {
+    int s = 0;
 #pragma unroll
-  for (int i = 1; i < kMaxSub; ++i)
-    if (i < a.n_sub && blk >= a.sub[i].tile_start) s = i;
-  const SubClass sc = a.sub[s];
-  const int nb_all = sc.count * a.B;
+    for (int i = 1; i < kMaxSub; ++i)
+      if (i < a.n_sub && blk >= a.sub[i].tile_start) s = i;
+    sc = a.sub[s];
+  }
+  const int nb_all = sc.count * p_B;
   const int q0 = (blk - sc.tile_start) * sc.window;
   if (q0 >= nb_all) return;
   const int nb = min(sc.window, nb_all - q0);
 
-  const int fi_lo = q0 / a.B;
+  const int fi_lo = q0 / p_B;
   using Sum = typename SumOf<IdxT>::type;
 
   // Bag q0 + i of the window: where it sits in the offsets (or lengths) array.
   auto bag_of = [&](int i, int& fi, int& b) -> int64_t {
     const int q = q0 + i;
-    fi = q / a.B;
-    b = q - fi * a.B;
-    return (int64_t)feat_key_pos(a, sc, fi) * a.B + b;
+    fi = q / p_B;
+    b = q - fi * p_B;
+    return (int64_t)feat_key_pos(a, sc, fi) * p_B + b;
   };
   // The first bag of every thread is requested before anything else: the
   // barrier below waits for outstanding loads, and this way the bag bounds
@@ -1006,14 +1020,14 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   if ((int)threadIdx.x < nb) {
     int fi, b;
     const int64_t bag = bag_of(threadIdx.x, fi, b);
-    first_lo = reinterpret_cast<const IdxT*>(a.offsets)[bag];
-    if (!FROM_LENGTHS) first_hi = reinterpret_cast<const IdxT*>(a.offsets)[bag + 1];
+    first_lo = reinterpret_cast<const IdxT*>(p_offsets)[bag];
+    if (!FROM_LENGTHS) first_hi = reinterpret_cast<const IdxT*>(p_offsets)[bag + 1];
   }
   // Descriptors of the features this window touches, kept in LDS so that a
   // round does not start with two dependent global loads.
   {
-    const int nfeat = min((q0 + nb - 1) / a.B - fi_lo + 1, kMaxWinFeat);
-    if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = a.cdescs[sc.first + fi_lo + threadIdx.x];
+    const int nfeat = min((q0 + nb - 1) / p_B - fi_lo + 1, kMaxWinFeat);
+    if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = p_cdescs[sc.first + fi_lo + threadIdx.x];
   }
   // From lengths: the total of everything in front of the window.  Its loads
   // go out after the window's own (loads return in order: whatever is waited
@@ -1021,8 +1035,8 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
   // below needs the sum.
   PrefixSum<IdxT> front_sum;
   if (FROM_LENGTHS)
-    front_sum.start(reinterpret_cast<const IdxT*>(a.offsets),
-                    (int64_t)feat_key_pos(a, sc, fi_lo) * a.B + (q0 - fi_lo * a.B));
+    front_sum.start(reinterpret_cast<const IdxT*>(p_offsets),
+                    (int64_t)feat_key_pos(a, sc, fi_lo) * p_B + (q0 - fi_lo * p_B));
   if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
   lds_barrier();
   TRA_STAMP(6);
@@ -1035,10 +1049,10 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
       // Kept as given: bag starts are the running sum of the lengths as they
       // are (what a separate cumsum would produce); a negative length only
       // makes its own bag empty.
-      len = (int)(first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag));
+      len = (int)(first ? (int64_t)first_lo : load_index<IdxT>(p_offsets, bag));
     } else {
-      const int64_t st = first ? (int64_t)first_lo : load_index<IdxT>(a.offsets, bag);
-      const int64_t en = first ? (int64_t)first_hi : load_index<IdxT>(a.offsets, bag + 1);
+      const int64_t st = first ? (int64_t)first_lo : load_index<IdxT>(p_offsets, bag);
+      const int64_t en = first ? (int64_t)first_hi : load_index<IdxT>(p_offsets, bag + 1);
       s_start[i] = st;
       len = max(0, (int)(en - st));
     }
@@ -1082,7 +1096,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
     // The window covers bags of features fi_lo .. fi_hi of the sub-class.  A
     // feature's bags are contiguous in `lengths`; where the next feature's
     // key position follows directly, the run simply continues.
-    const int fi_hi = (q0 + nb - 1) / a.B;
+    const int fi_hi = (q0 + nb - 1) / p_B;
     bool one_run = true;
     if (sc.key0 < 0)
       for (int fi = fi_lo; fi < fi_hi; ++fi) one_run = one_run && feat_key_pos(a, sc, fi + 1) == feat_key_pos(a, sc, fi) + 1;
@@ -1100,12 +1114,12 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const LookupA
       int64_t adj = (int64_t)front;  // start = adj + scan value, for the current run
       int64_t next_pos = -1;
       for (int fi = fi_lo; fi <= fi_hi; ++fi) {
-        const int first = max(0, fi * a.B - q0);        // first bag of this feature in the window
-        const int last = min(nb, (fi + 1) * a.B - q0);  // one past its last bag
-        const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * a.B + (q0 + first - fi * a.B);
+        const int first = max(0, fi * p_B - q0);        // first bag of this feature in the window
+        const int last = min(nb, (fi + 1) * p_B - q0);  // one past its last bag
+        const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * p_B + (q0 + first - fi * p_B);
         if (fi != fi_lo && pos != next_pos) {
           PrefixSum<IdxT> again;
-          again.start(reinterpret_cast<const IdxT*>(a.offsets), pos);
+          again.start(reinterpret_cast<const IdxT*>(p_offsets), pos);
           const Sum w_ = wave_last(wave_scan_incl(again.finish()));
           if (ln == 0) s_red[wv] = w_;
           lds_barrier();
@@ -1293,10 +1307,10 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
   do {                                                                                         \
     if (p.balanced && p.from_lengths)                                                          \
       hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, 4, true>), g,               \
-                         dim3(kCuThreads), p.lds_bytes, stream, a);                            \
+                         dim3(kCuThreads), p.lds_bytes, stream, a.offsets, a.cdescs, a.B, a.xcd_blocks, a.xcd_count, a.n_sub, a.sub[0].window, a.sub[0].count, a.sub[0].key0, a);                            \
     else if (p.balanced)                                                                       \
       hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kCuThreads),   \
-                         p.lds_bytes, stream, a);                                              \
+                         p.lds_bytes, stream, a.offsets, a.cdescs, a.B, a.xcd_blocks, a.xcd_count, a.n_sub, a.sub[0].window, a.sub[0].count, a.sub[0].key0, a);                                              \
     else if (p.from_lengths)                                                                   \
       hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, 4, true>), g,                  \
                          dim3(kBlockThreads), 0, stream, a);                                   \
