@@ -446,6 +446,37 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         ``position_weights`` (not an argument of the reference; the
         feature-processed subclass passes it) weighs every id by its position
         in its bag inside the lookup kernel, see the operator's ``forward``."""
+        # The common serving call first: one lookup operator, no weights, a KJT
+        # built from lengths whose keys are this module's features in order.
+        # Everything the general route below would establish is checked here
+        # in a few attribute reads, and the operator is launched directly.
+        ops_ = self._emb_modules
+        if len(ops_) == 1 and not self._is_weighted and position_weights is None and features._offsets is None:
+            op = ops_[0]
+            v, ln, keys = features._values, features._lengths, features._keys
+            if (
+                ln is not None
+                and (keys is self._feature_names or keys == self._feature_names)
+                and v.is_cuda
+                and ln.is_cuda
+                and (v.dtype is torch.int64 or v.dtype is torch.int32)
+                and ln.dtype is v.dtype
+                and ln.dim() == 1
+                and v.is_contiguous()
+                and ln.is_contiguous()
+                and op._weights_initialized
+                and v.device == op.current_device
+                and op._buffers["weights_dev"].device == v.device
+                and not getattr(self, MODULE_ATTR_CACHE_FEATURES_ORDER, False)
+            ):
+                K = len(keys)
+                B = ln.numel() // K if K else 0
+                if B > 0 and ln.numel() == K * B:
+                    out = torch.empty(B, self._total_D, dtype=self._output_dtype, device=v.device)
+                    op._launch_from_lengths(
+                        None, v, ln, int(v.dtype is torch.int64), None, B, K, v.numel(), out.data_ptr(), out.stride(0)
+                    )
+                    return KeyedTensor(keys=self._embedding_names, values=out, length_per_key=self._length_per_key)
         order = self._resolve_order(_get_kjt_keys(features))
         B = features.stride()
         indices = features.values()

@@ -33,6 +33,7 @@ from torchrec_amd.tbe.enums import BoundsCheckMode, EmbeddingLocation, PoolingMo
 _ENV_BOUNDS_CHECK = os.environ.get("TORCHREC_AMD_BOUNDS_CHECK", "0") == "1"
 _INT_DTYPES = (torch.int32, torch.int64)
 _BOUNDS_FATAL = int(BoundsCheckMode.FATAL)
+_FORWARD_LENGTHS = None  # the library's tra_tbe_forward_lengths, bound on first use
 
 _SUPPORTED_WEIGHTS = (SparseType.FP32, SparseType.FP16, SparseType.INT8, SparseType.INT4, SparseType.INT2)
 _TABLE_ALIGNMENT = 256
@@ -149,6 +150,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self._num_keys: Dict[Tuple[int, ...], int] = {}
         self._workspace: Dict[int, Tensor] = {}  # per stream: scratch of forward(offsets=None, lengths=...)
         self._ws_bytes: Dict[Tuple[int, int, int], int] = {}  # size of that scratch per (keys, batch size, id width)
+        self._ws_ptr: Dict[Tuple[int, int, int, int], int] = {}  # its address per (keys, batch size, id width, stream)
         self._weights_initialized = False
         self.weight_initialized = False
         self.register_buffer("weights_dev", torch.empty(0, dtype=torch.uint8, device=device), persistent=False)
@@ -175,6 +177,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             self.current_device = dev
             self._drop_plan()
             self._workspace.clear()
+            self._ws_ptr.clear()
         return self
 
     def _num_keys_of(self, positions: Tuple[int, ...]) -> int:
@@ -266,6 +269,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         state = self.__dict__.copy()
         state["_plans"] = {}
         state["_workspace"] = {}
+        state["_ws_ptr"] = {}
         return state
 
     def _get_plan(self, feature_positions: Optional[Tuple[int, ...]] = None) -> ctypes.c_void_p:
@@ -429,22 +433,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 )
             )
         elif offsets is None:
-            ws_key = (k_total, B, i64)
-            ws_bytes = self._ws_bytes.get(ws_key)
-            if ws_bytes is None:
-                ws_bytes = self._ws_bytes[ws_key] = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
-            stream = _lib.current_stream(dev)
-            # one scratch buffer per stream: calls queued on different streams must not share it
-            ws = self._workspace.get(stream)
-            if ws is None or ws.numel() < ws_bytes or ws.device != dev:
-                ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
-            _lib.check(
-                _lib.lib().tra_tbe_forward_lengths(
-                    self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices), _lib.ptr(lengths),
-                    i64, _lib.ptr(psw), B, k_total, L, int(self.pooling_mode),
-                    self.output_dtype, out_ptr, out_stride, ws.data_ptr(), stream,
-                )
-            )
+            self._launch_from_lengths(positions, indices, lengths, i64, psw, B, k_total, L, out_ptr, out_stride)
+            return out
         else:
             _lib.check(
                 _lib.lib().tra_tbe_forward(
@@ -458,6 +448,53 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             if bad:
                 raise IndexError(f"{bad} embedding indices were out of range")
         return out
+
+    def _launch_from_lengths(
+        self,
+        positions: Optional[Tuple[int, ...]],
+        indices: Tensor,
+        lengths: Tensor,
+        i64: int,
+        psw: Optional[Tensor],
+        B: int,
+        k_total: int,
+        L: int,
+        out_ptr: int,
+        out_stride: int,
+    ) -> None:
+        """The launch of ``forward(offsets=None, lengths=...)``.  The caller has checked the arguments:
+        contiguous device tensors on this operator's GPU, ``lengths`` of the ids' type with ``k_total * B``
+        entries, ``psw`` fp32 or None."""
+        dev = self.current_device
+        stream = _lib.current_stream(dev)
+        # The scratch buffer of this call shape on this stream (one per stream: calls queued on
+        # different streams must not share it), found again by one dictionary lookup.
+        ws_key = (k_total, B, i64, stream)
+        ws_ptr = self._ws_ptr.get(ws_key)
+        if ws_ptr is None:
+            ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
+            ws = self._workspace.get(stream)
+            if ws is None or ws.numel() < ws_bytes or ws.device != dev:
+                ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+                # a larger buffer replaced the stream's old one: forget the addresses handed out from it
+                for k in [k for k in self._ws_ptr if k[3] == stream]:
+                    del self._ws_ptr[k]
+            ws_ptr = self._ws_ptr[ws_key] = ws.data_ptr()
+        global _FORWARD_LENGTHS
+        fn = _FORWARD_LENGTHS
+        if fn is None:
+            fn = _FORWARD_LENGTHS = _lib.lib().tra_tbe_forward_lengths
+        rc = fn(
+            self._get_plan(positions), self._buffers["weights_dev"].data_ptr(), indices.data_ptr(),
+            lengths.data_ptr(), i64, None if psw is None else psw.data_ptr(), B, k_total, L,
+            int(self.pooling_mode), self.output_dtype, out_ptr, out_stride, ws_ptr, stream,
+        )
+        if rc != 0:
+            _lib.check(rc)
+        if _ENV_BOUNDS_CHECK or self.bounds_check_mode_int == _BOUNDS_FATAL:
+            bad = self.out_of_range_count()
+            if bad:
+                raise IndexError(f"{bad} embedding indices were out of range")
 
     def out_of_range_count(self) -> int:
         """Ids outside [0, rows) (other than -1) seen since the last call.  Synchronizes."""
