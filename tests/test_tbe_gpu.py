@@ -779,12 +779,17 @@ def test_padded_id_buffer(tuning, route):
     assert tbe.out_of_range_count() == 0
 
 
+@pytest.mark.parametrize("window", [None, 256, 100])
 @pytest.mark.parametrize("B,idt", [(8192, np.int32), (4096, np.int64)])
-def test_forward_from_lengths_long_prefix(B, idt):
+def test_forward_from_lengths_long_prefix(tuning, B, idt, window):
     """Enough bags that the blocks of the last windows sum the lengths in front
     of them in many batches of loads (26 x 8192 int32 lengths, 26 x 4096 int64
     ones): lengths entry == offsets entry, bit for bit, and the launch really
-    is the from-lengths one."""
+    is the from-lengths one.  Default windows (several hundred bags: staged by
+    the whole block) and forced small ones (staged by the block's first wave
+    while the other waves sum the prefix, here up to 850 KB of it)."""
+    if window is not None:
+        tuning(balanced=1, window=window)
     rng = np.random.default_rng(77 + B)
     T, rows, dim = 26, 20_000, 64
     tbe, store = build(rng, [(O.INT8, rows, dim)] * T, list(range(T)), O.MEAN, O.FP32, 16)

@@ -818,6 +818,61 @@ struct PrefixSum {
   }
 };
 
+// The same sum for waves that have nothing else in flight: the number of loads
+// follows the length of the range (in steps of four per thread), and all of
+// them are requested before the first is waited for.
+template <typename IdxT>
+struct PrefixSumAtOnce {
+  using S = typename SumOf<IdxT>::type;
+  static constexpr int V = 16 / (int)sizeof(IdxT);
+  struct __align__(16) Vec { IdxT v[V]; };
+  const Vec* vin;
+  int tid, nt, nvec, last;
+
+  template <int N>
+  __device__ __forceinline__ S steps(int k0) const {
+    Vec x[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) x[k] = vin[min((k0 + k) * nt + tid, last)];
+    S part = 0;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      S sum = 0;
+#pragma unroll
+      for (int i = 0; i < V; ++i) sum += (S)x[k].v[i];
+      part += (k0 + k) * nt + tid < nvec ? sum : (S)0;
+    }
+    return part;
+  }
+  // This thread's share of sum(lengths[0 .. p)); thread tid_ of nt_.
+  __device__ __forceinline__ S run(const IdxT* __restrict__ lengths, int64_t p, int tid_, int nt_) {
+    tid = tid_;
+    nt = nt_;
+    vin = reinterpret_cast<const Vec*>(lengths);
+    nvec = (int)(p / V);
+    last = max(nvec - 1, 0);
+    const int nk = (nvec + nt - 1) / nt;
+    // the elements after the last whole 16-byte step: one per thread
+    const int64_t rest = p - (int64_t)nvec * V;
+    const int64_t ti = (int64_t)nvec * V + min((int64_t)tid, max(rest - 1, (int64_t)0));
+    IdxT tail = lengths[max(min(ti, p - 1), (int64_t)0)];
+    if ((int64_t)tid >= rest) tail = 0;
+    S part = 0;
+    int k0 = 0;
+    for (; nk - k0 > 16; k0 += 16) part += steps<16>(k0);
+    const int r = nk - k0;
+    if (r > 12)
+      part += steps<16>(k0);
+    else if (r > 8)
+      part += steps<12>(k0);
+    else if (r > 4)
+      part += steps<8>(k0);
+    else if (r > 0)
+      part += steps<4>(k0);
+    return part + (S)tail;
+  }
+};
+
 // Inclusive scan over the 64 lanes of a wave.  32-bit sums use the data-parallel
 // lane moves of the VALU (shifts inside each row of 16 lanes, then lane 15 and
 // lane 31 broadcast into the following rows): six adds, no trip through the LDS
@@ -848,6 +903,11 @@ __device__ __forceinline__ int64_t wave_last(int64_t v) { return __shfl(v, kWave
 // every outstanding global load of the wave; the window kernel's prologue keeps
 // loads in flight across its barriers (nothing there is handed from wave to
 // wave through global memory).
+// The same inside one wave: LDS writes of its lanes are visible to its other lanes.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront", "local");
+  __builtin_amdgcn_wave_barrier();
+}
 __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
@@ -1013,154 +1073,245 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const void* p
     b = q - fi * p_B;
     return (int64_t)feat_key_pos(a, sc, fi) * p_B + b;
   };
-  // The first bag of every thread is requested before anything else: the
-  // barrier below waits for outstanding loads, and this way the bag bounds
-  // and the descriptors share one memory latency instead of queueing up.
-  IdxT first_lo = 0, first_hi = 0;
-  if ((int)threadIdx.x < nb) {
-    int fi, b;
-    const int64_t bag = bag_of(threadIdx.x, fi, b);
-    first_lo = reinterpret_cast<const IdxT*>(p_offsets)[bag];
-    if (!FROM_LENGTHS) first_hi = reinterpret_cast<const IdxT*>(p_offsets)[bag + 1];
-  }
-  // Descriptors of the features this window touches, kept in LDS so that a
-  // round does not start with two dependent global loads.
-  {
-    const int nfeat = min((q0 + nb - 1) / p_B - fi_lo + 1, kMaxWinFeat);
-    if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = p_cdescs[sc.first + fi_lo + threadIdx.x];
-  }
-  // From lengths: the total of everything in front of the window.  Its loads
-  // go out after the window's own (loads return in order: whatever is waited
-  // for first has to be issued first) and stay in flight until the scan
-  // below needs the sum.
-  PrefixSum<IdxT> front_sum;
-  if (FROM_LENGTHS)
-    front_sum.start(reinterpret_cast<const IdxT*>(p_offsets),
-                    (int64_t)feat_key_pos(a, sc, fi_lo) * p_B + (q0 - fi_lo * p_B));
-  if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
-  lds_barrier();
-  TRA_STAMP(6);
-  for (int i = threadIdx.x; i < nb; i += kCuThreads) {
-    int fi, b;
-    const int64_t bag = bag_of(i, fi, b);
-    const bool first = i == (int)threadIdx.x;
-    int len;
-    if (FROM_LENGTHS) {
-      // Kept as given: bag starts are the running sum of the lengths as they
-      // are (what a separate cumsum would produce); a negative length only
-      // makes its own bag empty.
-      len = (int)(first ? (int64_t)first_lo : load_index<IdxT>(p_offsets, bag));
-    } else {
-      const int64_t st = first ? (int64_t)first_lo : load_index<IdxT>(p_offsets, bag);
-      const int64_t en = first ? (int64_t)first_hi : load_index<IdxT>(p_offsets, bag + 1);
-      s_start[i] = st;
-      len = max(0, (int)(en - st));
-    }
-    s_len[i] = len;
-    s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
-    s_slot[i] = (uint16_t)atomicAdd(&s_hist[length_bin(len)], 1);
-  }
-  lds_barrier();
-  TRA_STAMP(7);
-  if (FROM_LENGTHS) {
-    __shared__ Sum s_red[kCuWaves];
-    __shared__ Sum s_wave_tot[kCuWaves];
-    const int t = threadIdx.x;
-    const int wv = t / kWaveSize;
-    const int ln = t & (kWaveSize - 1);
-    // Exclusive scan of the window's lengths (window order): two bags per
-    // thread, wave scan, then the 16 wave totals.  The same barrier carries
-    // the block-wide total of everything in front of the window.
-    // (Only the waves that hold bags scan; every instruction that all 16 waves
-    // of the block execute costs 16 issue cycles per SIMD.)
-    const bool holds_bags = 2 * wv * kWaveSize < nb;
-    Sum x0 = 0, x1 = 0, inc = 0;
-    if (holds_bags) {
-      x0 = 2 * t < nb ? s_len[2 * t] : 0;
-      x1 = 2 * t + 1 < nb ? s_len[2 * t + 1] : 0;
-      inc = wave_scan_incl((Sum)(x0 + x1));
-    }
-    const Sum front_w = wave_last(wave_scan_incl(front_sum.finish()));
-    if (ln == kWaveSize - 1) s_wave_tot[wv] = inc;
-    if (ln == 0) s_red[wv] = front_w;
-    lds_barrier();
-    Sum before = 0, front = 0;
+  // What a bag's start in LDS still lacks (from lengths, small windows: the sum
+  // of everything in front of the window arrives last and is added on reading).
+  Sum front_add = 0;
+  __shared__ Sum s_red[kCuWaves];
+  // A window of at most 4 x 64 bags is staged, scanned and ranked by the
+  // block's first wave alone, four consecutive bags per lane, with no block
+  // barrier on the way; from lengths, the other fifteen waves meanwhile sum
+  // the lengths in front of the window.  One barrier joins the two.
+  const bool solo = FROM_LENGTHS && nb <= 4 * kWaveSize && sc.key0 >= 0;
+  if (solo) {
+    const int wv = threadIdx.x / kWaveSize;
+    const int ln = threadIdx.x & (kWaveSize - 1);
+    if (wv == 0) {
+      IdxT given[4];  // lengths as they stand in the KJT (lanes past the window repeat its last bag)
+      int fis[4], bs[4];
 #pragma unroll
-    for (int w = 0; w < kCuWaves; ++w) front += s_red[w];
-    if (holds_bags) {
+      for (int k = 0; k < 4; ++k) {
+        const int64_t bag = bag_of(min(4 * ln + k, nb - 1), fis[k], bs[k]);
+        given[k] = reinterpret_cast<const IdxT*>(p_offsets)[bag];
+      }
+      {
+        const int nfeat = min((q0 + nb - 1) / p_B - fi_lo + 1, kMaxWinFeat);
+        if (ln < nfeat) s_desc[ln] = p_cdescs[sc.first + fi_lo + ln];
+      }
 #pragma unroll
-      for (int w = 0; w < kCuWaves; ++w)
-        if (w < wv) before += s_wave_tot[w];
-    }
-    const Sum excl = before + inc - (x0 + x1);
-    // The window covers bags of features fi_lo .. fi_hi of the sub-class.  A
-    // feature's bags are contiguous in `lengths`; where the next feature's
-    // key position follows directly, the run simply continues.
-    const int fi_hi = (q0 + nb - 1) / p_B;
-    bool one_run = true;
-    if (sc.key0 < 0)
-      for (int fi = fi_lo; fi < fi_hi; ++fi) one_run = one_run && feat_key_pos(a, sc, fi + 1) == feat_key_pos(a, sc, fi) + 1;
-    if (one_run) {
-      if (2 * t < nb) s_start[2 * t] = (int64_t)(front + excl);
-      if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(front + excl + x0);
-      lds_barrier();
-    } else {
-      // General case: keep the bare scan, then add to each run what lies in
-      // front of it (summed again for every run that does not continue the
-      // previous one).
-      if (2 * t < nb) s_start[2 * t] = (int64_t)excl;
-      if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(excl + x0);
-      lds_barrier();
-      int64_t adj = (int64_t)front;  // start = adj + scan value, for the current run
-      int64_t next_pos = -1;
-      for (int fi = fi_lo; fi <= fi_hi; ++fi) {
-        const int first = max(0, fi * p_B - q0);        // first bag of this feature in the window
-        const int last = min(nb, (fi + 1) * p_B - q0);  // one past its last bag
-        const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * p_B + (q0 + first - fi * p_B);
-        if (fi != fi_lo && pos != next_pos) {
-          PrefixSum<IdxT> again;
-          again.start(reinterpret_cast<const IdxT*>(p_offsets), pos);
-          const Sum w_ = wave_last(wave_scan_incl(again.finish()));
-          if (ln == 0) s_red[wv] = w_;
-          lds_barrier();
-          Sum total = 0;
+      for (int k = 0; k < kLenBins / kWaveSize; ++k) s_hist[ln + k * kWaveSize] = 0;
+      wave_lds_sync();
+      TRA_STAMP(6);
+      int len[4], slot[4];
+      Sum raw[4];
 #pragma unroll
-          for (int w = 0; w < kCuWaves; ++w) total += s_red[w];
-          adj = (int64_t)total - s_start[first];
+      for (int k = 0; k < 4; ++k) {
+        const int i = 4 * ln + k;
+        raw[k] = 0;
+        len[k] = 0;
+        slot[k] = 0;
+        if (i < nb) {
+          // Kept as given: bag starts are the running sum of the lengths as
+          // they are; a negative length only makes its own bag empty.
+          raw[k] = (Sum)given[k];
+          len[k] = (int)given[k];
+          s_len[i] = len[k];
+          s_ent[i] = ((uint32_t)fis[k] << kBagBits) | (uint32_t)bs[k];
+          slot[k] = atomicAdd(&s_hist[length_bin(len[k])], 1);
         }
-        next_pos = pos + (last - first);
-        lds_barrier();  // s_red and s_start[first] have been read by everyone
-        for (int i = first + t; i < last; i += kCuThreads) s_start[i] += adj;
+      }
+      // Bag starts inside the window: exclusive scan in window order.
+      const Sum tot = raw[0] + raw[1] + raw[2] + raw[3];
+      Sum run = wave_scan_incl(tot) - tot;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (4 * ln + k < nb) s_start[4 * ln + k] = (int64_t)run;
+        run += raw[k];
+      }
+      if (ln == 0) s_red[0] = 0;
+      wave_lds_sync();
+      TRA_STAMP(7);
+      TRA_STAMP(1);
+      {  // counting sort, longest first (as in the general route below)
+        int h[kLenBins / kWaveSize];
+        int sum = 0;
+#pragma unroll
+        for (int k = 0; k < kLenBins / kWaveSize; ++k) {
+          h[k] = s_hist[kLenBins - 1 - (ln * (kLenBins / kWaveSize) + k)];
+          sum += h[k];
+        }
+        const int incl = wave_scan_incl((int32_t)sum);
+        int base = incl - sum;
+#pragma unroll
+        for (int k = 0; k < kLenBins / kWaveSize; ++k) {
+          s_hist[kLenBins - 1 - (ln * (kLenBins / kWaveSize) + k)] = base;
+          base += h[k];
+        }
+      }
+      wave_lds_sync();
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (4 * ln + k < nb) s_order[s_hist[length_bin(len[k])] + slot[k]] = (uint16_t)(4 * ln + k);
+    } else {
+      PrefixSumAtOnce<IdxT> front_sum;
+      const Sum mine = front_sum.run(reinterpret_cast<const IdxT*>(p_offsets),
+                                     (int64_t)feat_key_pos(a, sc, fi_lo) * p_B + (q0 - fi_lo * p_B),
+                                     (int)threadIdx.x - kWaveSize, kCuThreads - kWaveSize);
+      const Sum front_w = wave_last(wave_scan_incl(mine));
+      if (ln == 0) s_red[wv] = front_w;
+    }
+    lds_barrier();
+#pragma unroll
+    for (int w = 0; w < kCuWaves; ++w) front_add += s_red[w];
+    TRA_STAMP(2);
+  } else {
+    // The first bag of every thread is requested before anything else: the
+    // barrier below waits for outstanding loads, and this way the bag bounds
+    // and the descriptors share one memory latency instead of queueing up.
+    IdxT first_lo = 0, first_hi = 0;
+    if ((int)threadIdx.x < nb) {
+      int fi, b;
+      const int64_t bag = bag_of(threadIdx.x, fi, b);
+      first_lo = reinterpret_cast<const IdxT*>(p_offsets)[bag];
+      if (!FROM_LENGTHS) first_hi = reinterpret_cast<const IdxT*>(p_offsets)[bag + 1];
+    }
+    // Descriptors of the features this window touches, kept in LDS so that a
+    // round does not start with two dependent global loads.
+    {
+      const int nfeat = min((q0 + nb - 1) / p_B - fi_lo + 1, kMaxWinFeat);
+      if ((int)threadIdx.x < nfeat) s_desc[threadIdx.x] = p_cdescs[sc.first + fi_lo + threadIdx.x];
+    }
+    // From lengths: the total of everything in front of the window.  Its loads
+    // go out after the window's own (loads return in order: whatever is waited
+    // for first has to be issued first) and stay in flight until the scan
+    // below needs the sum.
+    PrefixSum<IdxT> front_sum;
+    if (FROM_LENGTHS)
+      front_sum.start(reinterpret_cast<const IdxT*>(p_offsets),
+                      (int64_t)feat_key_pos(a, sc, fi_lo) * p_B + (q0 - fi_lo * p_B));
+    if (threadIdx.x < kLenBins) s_hist[threadIdx.x] = 0;
+    lds_barrier();
+    TRA_STAMP(6);
+    for (int i = threadIdx.x; i < nb; i += kCuThreads) {
+      int fi, b;
+      const int64_t bag = bag_of(i, fi, b);
+      const bool first = i == (int)threadIdx.x;
+      int len;
+      if (FROM_LENGTHS) {
+        // Kept as given: bag starts are the running sum of the lengths as they
+        // are (what a separate cumsum would produce); a negative length only
+        // makes its own bag empty.
+        len = (int)(first ? (int64_t)first_lo : load_index<IdxT>(p_offsets, bag));
+      } else {
+        const int64_t st = first ? (int64_t)first_lo : load_index<IdxT>(p_offsets, bag);
+        const int64_t en = first ? (int64_t)first_hi : load_index<IdxT>(p_offsets, bag + 1);
+        s_start[i] = st;
+        len = max(0, (int)(en - st));
+      }
+      s_len[i] = len;
+      s_ent[i] = ((uint32_t)fi << kBagBits) | (uint32_t)b;
+      s_slot[i] = (uint16_t)atomicAdd(&s_hist[length_bin(len)], 1);
+    }
+    lds_barrier();
+    TRA_STAMP(7);
+    if (FROM_LENGTHS) {
+      __shared__ Sum s_wave_tot[kCuWaves];
+      const int t = threadIdx.x;
+      const int wv = t / kWaveSize;
+      const int ln = t & (kWaveSize - 1);
+      // Exclusive scan of the window's lengths (window order): two bags per
+      // thread, wave scan, then the 16 wave totals.  The same barrier carries
+      // the block-wide total of everything in front of the window.
+      // (Only the waves that hold bags scan; every instruction that all 16 waves
+      // of the block execute costs 16 issue cycles per SIMD.)
+      const bool holds_bags = 2 * wv * kWaveSize < nb;
+      Sum x0 = 0, x1 = 0, inc = 0;
+      if (holds_bags) {
+        x0 = 2 * t < nb ? s_len[2 * t] : 0;
+        x1 = 2 * t + 1 < nb ? s_len[2 * t + 1] : 0;
+        inc = wave_scan_incl((Sum)(x0 + x1));
+      }
+      const Sum front_w = wave_last(wave_scan_incl(front_sum.finish()));
+      if (ln == kWaveSize - 1) s_wave_tot[wv] = inc;
+      if (ln == 0) s_red[wv] = front_w;
+      lds_barrier();
+      Sum before = 0, front = 0;
+#pragma unroll
+      for (int w = 0; w < kCuWaves; ++w) front += s_red[w];
+      if (holds_bags) {
+#pragma unroll
+        for (int w = 0; w < kCuWaves; ++w)
+          if (w < wv) before += s_wave_tot[w];
+      }
+      const Sum excl = before + inc - (x0 + x1);
+      // The window covers bags of features fi_lo .. fi_hi of the sub-class.  A
+      // feature's bags are contiguous in `lengths`; where the next feature's
+      // key position follows directly, the run simply continues.
+      const int fi_hi = (q0 + nb - 1) / p_B;
+      bool one_run = true;
+      if (sc.key0 < 0)
+        for (int fi = fi_lo; fi < fi_hi; ++fi) one_run = one_run && feat_key_pos(a, sc, fi + 1) == feat_key_pos(a, sc, fi) + 1;
+      if (one_run) {
+        if (2 * t < nb) s_start[2 * t] = (int64_t)(front + excl);
+        if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(front + excl + x0);
         lds_barrier();
+      } else {
+        // General case: keep the bare scan, then add to each run what lies in
+        // front of it (summed again for every run that does not continue the
+        // previous one).
+        if (2 * t < nb) s_start[2 * t] = (int64_t)excl;
+        if (2 * t + 1 < nb) s_start[2 * t + 1] = (int64_t)(excl + x0);
+        lds_barrier();
+        int64_t adj = (int64_t)front;  // start = adj + scan value, for the current run
+        int64_t next_pos = -1;
+        for (int fi = fi_lo; fi <= fi_hi; ++fi) {
+          const int first = max(0, fi * p_B - q0);        // first bag of this feature in the window
+          const int last = min(nb, (fi + 1) * p_B - q0);  // one past its last bag
+          const int64_t pos = (int64_t)feat_key_pos(a, sc, fi) * p_B + (q0 + first - fi * p_B);
+          if (fi != fi_lo && pos != next_pos) {
+            PrefixSum<IdxT> again;
+            again.start(reinterpret_cast<const IdxT*>(p_offsets), pos);
+            const Sum w_ = wave_last(wave_scan_incl(again.finish()));
+            if (ln == 0) s_red[wv] = w_;
+            lds_barrier();
+            Sum total = 0;
+#pragma unroll
+            for (int w = 0; w < kCuWaves; ++w) total += s_red[w];
+            adj = (int64_t)total - s_start[first];
+          }
+          next_pos = pos + (last - first);
+          lds_barrier();  // s_red and s_start[first] have been read by everyone
+          for (int i = first + t; i < last; i += kCuThreads) s_start[i] += adj;
+          lds_barrier();
+        }
       }
     }
-  }
-  TRA_STAMP(1);
-  // Counting sort, longest first: a permutation of 0..nb-1.  hist[] holds the
-  // bin sizes and every bag already has its slot within its bin; one wave
-  // turns the sizes into start positions (bins in descending order).
-  if (threadIdx.x < kWaveSize) {
-    const int l = threadIdx.x;
-    int h[kLenBins / kWaveSize];
-    int sum = 0;
+    TRA_STAMP(1);
+    // Counting sort, longest first: a permutation of 0..nb-1.  hist[] holds the
+    // bin sizes and every bag already has its slot within its bin; one wave
+    // turns the sizes into start positions (bins in descending order).
+    if (threadIdx.x < kWaveSize) {
+      const int l = threadIdx.x;
+      int h[kLenBins / kWaveSize];
+      int sum = 0;
 #pragma unroll
-    for (int k = 0; k < kLenBins / kWaveSize; ++k) {
-      h[k] = s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)];
-      sum += h[k];
-    }
-    const int incl = wave_scan_incl((int32_t)sum);
-    int base = incl - sum;
+      for (int k = 0; k < kLenBins / kWaveSize; ++k) {
+        h[k] = s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)];
+        sum += h[k];
+      }
+      const int incl = wave_scan_incl((int32_t)sum);
+      int base = incl - sum;
 #pragma unroll
-    for (int k = 0; k < kLenBins / kWaveSize; ++k) {
-      s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)] = base;
-      base += h[k];
+      for (int k = 0; k < kLenBins / kWaveSize; ++k) {
+        s_hist[kLenBins - 1 - (l * (kLenBins / kWaveSize) + k)] = base;
+        base += h[k];
+      }
     }
+    lds_barrier();
+    for (int i = threadIdx.x; i < nb; i += kCuThreads)
+      s_order[s_hist[length_bin(s_len[i])] + s_slot[i]] = (uint16_t)i;
+    lds_barrier();
+    TRA_STAMP(2);
   }
-  lds_barrier();
-  for (int i = threadIdx.x; i < nb; i += kCuThreads)
-    s_order[s_hist[length_bin(s_len[i])] + s_slot[i]] = (uint16_t)i;
-  lds_barrier();
-  TRA_STAMP(2);
 
   const int lane = threadIdx.x & (kWaveSize - 1);
   const int wave = threadIdx.x / kWaveSize;
@@ -1186,7 +1337,7 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const void* p
     const int fi = (int)(ent >> kBagBits);
     const int b = (int)(ent & ((1u << kBagBits) - 1));
     const FeatureDesc d = fi - fi_lo < kMaxWinFeat ? s_desc[fi - fi_lo] : a.cdescs[sc.first + fi];
-    const int64_t start = s_start[i];
+    const int64_t start = s_start[i] + (int64_t)front_add;
     const int len = active ? max(s_len[i], 0) : 0;
     // The round's trip count.  Lengths below 192 have a sort bin each, so
     // the round's first bag is its longest; from 192 up a bin holds a range of
