@@ -244,6 +244,72 @@ def test_qebc_kjt_from_lengths_equals_from_offsets():
     assert torch.isfinite(a.values()).all()
 
 
+def test_qebc_short_host_route_and_what_falls_back():
+    """forward() takes a short route for the common serving call (one unweighted
+    operator, KJT from lengths, keys in module order, contiguous device tensors
+    of one integer type).  Its result, and the result of every input that must
+    not take it (other key order, a superset of keys, lengths of another integer
+    type, non-contiguous ids, a KJT that already holds offsets, the
+    cache-features-order flag), against the general route fed with offsets."""
+    torch.manual_seed(11)
+    T, B = 4, 50
+    tables = [EmbeddingBagConfig(name=f"t{t}", embedding_dim=64, num_embeddings=300 + t, feature_names=[f"f{t}"],
+                                 data_type=DataType.INT8, pooling=PoolingType.MEAN if t % 2 else PoolingType.SUM)
+              for t in range(T)]
+    # one pooling type per module so that it is a single operator
+    tables = [EmbeddingBagConfig(name=c.name, embedding_dim=c.embedding_dim, num_embeddings=c.num_embeddings,
+                                 feature_names=c.feature_names, data_type=c.data_type, pooling=PoolingType.SUM)
+              for c in tables]
+    m = QuantEBC(tables, False, DEV, output_dtype=torch.half)
+    assert len(m._emb_modules) == 1
+    tbe = m._emb_modules[0]
+    tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, device=DEV))
+    for t in range(T):
+        tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+    keys = [f"f{t}" for t in range(T)]
+    lengths = torch.randint(0, 7, (T * B,), dtype=torch.int64, device=DEV)
+    values = torch.randint(0, 300, (int(lengths.sum()),), dtype=torch.int64, device=DEV)
+    offsets = torch.zeros(T * B + 1, dtype=torch.int64, device=DEV)
+    offsets[1:] = torch.cumsum(lengths, 0)
+    want = m(KeyedJaggedTensor(keys=keys, values=values, offsets=offsets)).values()
+
+    def same(kjt, module=m):
+        got = module(kjt)
+        assert got.keys() == keys
+        assert torch.equal(got.values().view(torch.int16), want.view(torch.int16))
+
+    same(KeyedJaggedTensor(keys=keys, values=values, lengths=lengths))            # the short route
+    same(KeyedJaggedTensor(keys=list(keys), values=values, lengths=lengths))      # an equal list, not the same object
+    same(KeyedJaggedTensor(keys=keys, values=values, lengths=lengths.to(torch.int32)))  # lengths of another type
+    wide = torch.stack([values, values + 1], dim=1)
+    assert not wide[:, 0].is_contiguous()
+    same(KeyedJaggedTensor(keys=keys, values=wide[:, 0], lengths=lengths))        # strided ids
+    kjt = KeyedJaggedTensor(keys=keys, values=values, lengths=lengths)
+    kjt.offsets()                                                                 # offsets already derived
+    same(kjt)
+    # other key order, and a superset of the keys
+    perm = [2, 0, 3, 1]
+    Lm = lengths.view(T, B)
+    seg = [values[offsets[t * B]:offsets[(t + 1) * B]] for t in range(T)]
+    extra = torch.randint(0, 5, (B,), dtype=torch.int64, device=DEV)
+    same(KeyedJaggedTensor(keys=[keys[p] for p in perm], values=torch.cat([seg[p] for p in perm]),
+                           lengths=torch.cat([Lm[p] for p in perm])))
+    same(KeyedJaggedTensor(keys=["other"] + keys, lengths=torch.cat([extra, lengths]),
+                           values=torch.cat([torch.zeros(int(extra.sum()), dtype=torch.int64, device=DEV), values])))
+    # int32 throughout takes the short route as well
+    want32 = want
+    got32 = m(KeyedJaggedTensor(keys=keys, values=values.to(torch.int32), lengths=lengths.to(torch.int32))).values()
+    assert torch.equal(got32.view(torch.int16), want32.view(torch.int16))
+    # with the flag, the first key order seen is kept (the reference's contract): general route
+    m2 = QuantEBC(tables, False, DEV, output_dtype=torch.half, cache_features_order=True)
+    m2._emb_modules[0].weights_dev.copy_(tbe.weights_dev)
+    same(KeyedJaggedTensor(keys=keys, values=values, lengths=lengths), m2)
+    same(KeyedJaggedTensor(keys=keys, values=values, lengths=lengths), m2)
+    # a CPU KJT is refused by either route
+    with pytest.raises(Exception):
+        m(KeyedJaggedTensor(keys=keys, values=values.cpu(), lengths=lengths.cpu()))
+
+
 @pytest.mark.parametrize("from_lengths", [True, False])
 def test_forwards_in_flight_on_several_streams(from_lengths):
     """Independent requests on separate HIP streams (a serving loop): lookups of
