@@ -725,6 +725,7 @@ __device__ __forceinline__ void finish_bag(float (&acc)[NE], const LookupArgs& a
 #endif
 constexpr int kCuThreads = TRA_CU_THREADS;
 constexpr int kCuWaves = kCuThreads / kWaveSize;
+static_assert(kCuWaves >= 2, "the window kernel splits its prologue between the first wave and the others");
 constexpr int kMaxWindow = TRA_MAX_WINDOW;
 constexpr int kBagBits = 20;  // window entry = (feature index in sub-class << 20) | sample
 
