@@ -1024,7 +1024,10 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
 // and the block derives its bags' start positions itself: one block-wide sum
 // of everything in front of the window plus a scan of the window in LDS.
 template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, bool FROM_LENGTHS = false>
-__global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(const void* p_offsets, const FeatureDesc* p_cdescs, int32_t p_B, int32_t p_xcd_blocks, int32_t p_xcd_count, int32_t p_n_sub, int32_t p_window0, int32_t p_count0, int32_t p_key0, const LookupArgs a) {
+__global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(
+    const void* p_offsets, const FeatureDesc* p_cdescs, int32_t p_B, int32_t p_xcd_blocks,
+    int32_t p_xcd_count, int32_t p_n_sub, int32_t p_window0, int32_t p_count0, int32_t p_key0,
+    const LookupArgs a) {
   constexpr int NE = CB * 8 / Traits<DTYPE>::kBits;
   extern __shared__ unsigned char tra_dyn_smem[];  // only its size matters (one block per CU)
   __shared__ int64_t s_start[kMaxWindow];
@@ -1455,14 +1458,18 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
     hipLaunchKernelGGL((tbe_nobag_kernel<DTYPE, CB, IdxT>), g, dim3(kBlockThreads), 0, stream, a);
     return;
   }
+// What the window kernel's first fetches need, repeated as its leading parameters.
+#define TRA_CU_LEADING_ARGS                                                                   \
+  a.offsets, a.cdescs, a.B, a.xcd_blocks, a.xcd_count, a.n_sub, a.sub[0].window, a.sub[0].count, \
+      a.sub[0].key0
 #define TRA_POOLED(W, U)                                                                       \
   do {                                                                                         \
     if (p.balanced && p.from_lengths)                                                          \
       hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, 4, true>), g,               \
-                         dim3(kCuThreads), p.lds_bytes, stream, a.offsets, a.cdescs, a.B, a.xcd_blocks, a.xcd_count, a.n_sub, a.sub[0].window, a.sub[0].count, a.sub[0].key0, a);                            \
+                         dim3(kCuThreads), p.lds_bytes, stream, TRA_CU_LEADING_ARGS, a);       \
     else if (p.balanced)                                                                       \
       hipLaunchKernelGGL((tbe_pooled_cu_kernel<DTYPE, CB, IdxT, W, U>), g, dim3(kCuThreads),   \
-                         p.lds_bytes, stream, a.offsets, a.cdescs, a.B, a.xcd_blocks, a.xcd_count, a.n_sub, a.sub[0].window, a.sub[0].count, a.sub[0].key0, a);                                              \
+                         p.lds_bytes, stream, TRA_CU_LEADING_ARGS, a);                         \
     else if (p.from_lengths)                                                                   \
       hipLaunchKernelGGL((tbe_pooled_kernel<DTYPE, CB, IdxT, W, 4, true>), g,                  \
                          dim3(kBlockThreads), 0, stream, a);                                   \
@@ -1480,6 +1487,7 @@ void launch_typed(const LookupArgs& a, const LaunchParams& p, hipStream_t stream
     if (p.unroll >= 8) TRA_POOLED(kUnweighted, 8); else if (p.unroll >= 4) TRA_POOLED(kUnweighted, 4); else TRA_POOLED(kUnweighted, 2);
   }
 #undef TRA_POOLED
+#undef TRA_CU_LEADING_ARGS
 }
 
 template <int DTYPE, int CB>
