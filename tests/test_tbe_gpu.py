@@ -729,6 +729,43 @@ def test_small_call_from_lengths_one_launch(tuning, B, idt, pooling, weighted):
     assert tbe.out_of_range_count() == 0
 
 
+@pytest.mark.parametrize("pooling", [O.SUM, O.MEAN])
+def test_negative_lengths_same_on_every_route(tuning, pooling):
+    """A malformed KJT with a few negative lengths: bag starts are the running
+    sum of the lengths as they stand and a negative length makes its own bag
+    empty.  The same on every route a lengths call can take (scan + lookup, the
+    static kernel summing its own prefix, the window kernel staged by one wave
+    and by the whole block) and through the offsets entry fed with the running
+    sum: all outputs bit for bit equal."""
+    rng = np.random.default_rng(606 + pooling)
+    T, B, rows, dim = 3, 400, 500, 64
+    tbe, store = build(rng, [(O.INT4, rows, dim)] * T, list(range(T)), pooling, O.FP32, 16)
+    lengths = rng.integers(0, 12, T * B).astype(np.int32)
+    bad = rng.choice(np.arange(5, T * B - 5), 9, replace=False)
+    lengths[bad] = -rng.integers(1, 4, len(bad)).astype(np.int32)   # never below the running sum's start
+    offsets = np.zeros(T * B + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(lengths)
+    assert offsets.min() >= 0
+    ids = rng.integers(0, rows, int(offsets.max()) + 8).astype(np.int32)
+    ti = torch.from_numpy(ids).to(DEV)
+    tl = torch.from_numpy(lengths).to(DEV)
+    ref = tbe(ti, torch.from_numpy(offsets).to(DEV), batch_size=B).cpu().numpy()
+    empty_rows = ref.reshape(B, T, dim)[(bad % B), (bad // B)]
+    assert not empty_rows.any()                      # the negative bags pooled nothing
+    outs = {}
+    outs["static, own prefix"] = tbe(ti, None, lengths=tl, batch_size=B).cpu().numpy()
+    tuning(fused_scan=0)
+    outs["scan + lookup"] = tbe(ti, None, lengths=tl, batch_size=B).cpu().numpy()
+    tuning(fused_scan=None)
+    tuning(balanced=1, window=100)
+    outs["window, one wave stages"] = tbe(ti, None, lengths=tl, batch_size=B).cpu().numpy()
+    outs["window, offsets"] = tbe(ti, torch.from_numpy(offsets).to(DEV), batch_size=B).cpu().numpy()
+    tuning(window=300)
+    outs["window, block stages"] = tbe(ti, None, lengths=tl, batch_size=B).cpu().numpy()
+    for name, got in outs.items():
+        assert bits_equal(got, ref) == 0, name
+
+
 @pytest.mark.parametrize("T,B,route", [(1, 70_000, "offsets"), (1, 70_000, "lengths"), (2, 40_000, "lengths"),
                                        (1, 1_100_000, "offsets"), (1, 1_100_000, "lengths"),
                                        (300, 3, "offsets"), (300, 3, "lengths"), (300, 40, "lengths"),
