@@ -321,9 +321,11 @@ constexpr int kByPosition = 2;  // position weight of the id's place in its bag
 // its bag, or a bad id) is redirected to row 0 and flagged invalid; consume_row
 // then multiplies it away exactly.  Returns 1 for a bad id (out of range and
 // not -1).
-template <int DTYPE, int CB, int WEIGHTED, typename IdxT>
+// GIVEN_W: the caller already holds the row's weight (`given_w`), fetched a
+// lane group at a time like the ids; no weight load is issued here.
+template <int DTYPE, int CB, int WEIGHTED, typename IdxT, bool GIVEN_W = false>
 __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT last,
-                                          const LookupArgs& a, const RowWalk& w) {
+                                          const LookupArgs& a, const RowWalk& w, float given_w = 1.0f) {
   const uint8_t* lane_base = w.lane_base;  // table + this lane's chunk offset
   const int chunk_off = w.chunk_off;
   bool valid;
@@ -353,7 +355,9 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
       r.hdr = 0;
     r.d = load_chunk<CB>(chunk);
   }
-  if constexpr (WEIGHTED) {
+  if constexpr (WEIGHTED != 0 && GIVEN_W) {
+    r.w = given_w;
+  } else if constexpr (WEIGHTED) {
     using UIdxT = typename std::make_unsigned<IdxT>::type;
     if constexpr (WEIGHTED == kByPosition) {
       // The weight of this id's place in its bag, clamped into the feature's
@@ -570,8 +574,26 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     const int r = j * lpr_u + c;
     return fetch_id<IdxT>(a, r < len, start + (IdxT)r, last);
   };
+  // Weights travel the same way: lane c of the group loads the weight of id
+  // number j * lpr + c (per-sample weights: psw at that position; position
+  // weights: the table entry of that place in the bag), one load per lpr rows.
+  auto load_weights = [&](int j) -> float {
+    if constexpr (WEIGHTED == kPerSample) {
+      using UIdxT = typename std::make_unsigned<IdxT>::type;
+      const IdxT p = start + (IdxT)(j * lpr_u + c);
+      return a.psw[(UIdxT)p < (UIdxT)last ? p : last];
+    } else if constexpr (WEIGHTED == kByPosition) {
+      const uint32_t k = (uint32_t)(j * lpr_u + c);
+      const float v = w.pw[k < w.pw_last ? k : w.pw_last];
+      return w.pw_on ? v : 1.0f;
+    } else {
+      return 1.0f;
+    }
+  };
   IdxT cur = load_block(0);
   IdxT nxt = load_block(1);
+  float wcur = load_weights(0);
+  float wnxt = load_weights(1);
   int cur_j = 0;
   // Id of row r (wave-uniform), or -1 past the bag's end.  r lies in the
   // current block: a batch of U rows never straddles two blocks (U divides
@@ -582,12 +604,21 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     const int src = group_lane0 + (r - cur_j * lpr_u);
     return (IdxT)__shfl(cur, src, kWaveSize);
   };
+  auto weight_of = [&](int r) -> float {
+    if constexpr (WEIGHTED == 0) return 1.0f;
+    const int src = group_lane0 + (r - cur_j * lpr_u);
+    return __shfl(wcur, src, kWaveSize);
+  };
   // Entering the block of row rb: make it the current one and request the next.
   auto enter = [&](int rb) {
     const int j = rb / lpr_u;
     if (j > cur_j) {
       cur = nxt;
       nxt = load_block(j + 1);
+      if constexpr (WEIGHTED != 0) {
+        wcur = wnxt;
+        wnxt = load_weights(j + 1);
+      }
       cur_j = j;
     }
   };
@@ -596,12 +627,16 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     cur = nxt;
     ++cur_j;
     nxt = load_block(cur_j + 1);
+    if constexpr (WEIGHTED != 0) {
+      wcur = wnxt;
+      wnxt = load_weights(cur_j + 1);
+    }
   };
   RowBuf<CB> bufA[U], bufB[U];
   int bad = 0;
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(u), start + u, last, a, w);
+    bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT, true>(bufA[u], id_of(u), start + u, last, a, w, weight_of(u));
   int it = 0;
   if constexpr (TWO_BATCHES) {
     // Whole iterations (2 * U rows, all inside the longest bag) run without the
@@ -612,13 +647,13 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     for (; it + 2 * U <= max_len; it += 2 * U) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
+        bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT, true>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w, weight_of(it + U + u));
 #pragma unroll
       for (int u = 0; u < U; ++u) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u], w);
       advance();
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
+        bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT, true>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w, weight_of(it + 2 * U + u));
 #pragma unroll
       for (int u = 0; u < U; ++u) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u], w);
     }
@@ -627,7 +662,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     if constexpr (!TWO_BATCHES) enter(it + U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w);
+      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT, true>(bufB[u], id_of(it + U + u), start + it + U + u, last, a, w, weight_of(it + U + u));
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (it + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufA[u], w);
@@ -635,7 +670,7 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
     if constexpr (TWO_BATCHES) advance(); else enter(it + 2 * U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w);
+      bad += fetch_row<DTYPE, CB, WEIGHTED, IdxT, true>(bufA[u], id_of(it + 2 * U + u), start + it + 2 * U + u, last, a, w, weight_of(it + 2 * U + u));
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u], w);
