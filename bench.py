@@ -52,6 +52,9 @@ def parse_args():
                    help="also time the same steps dealt round-robin to this many HIP streams (independent "
                         "requests in flight); 0 or 1 = skip")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-pcie", action="store_true",
+                   help="skip the leg that feeds every step from pinned host memory (profiling runs: the kernel "
+                        "averages then cover launches with resident inputs only)")
     p.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline sample")
     p.add_argument("--rocprof-summary", metavar="DIR", default=None,
                    help="no benchmark: summarize rocprofv3 CSV output under DIR (kernel_stats / counter_collection) "
@@ -534,16 +537,18 @@ def main():
         n = src[0].numel()
         return module(KeyedJaggedTensor(keys=keys, values=v[:n], lengths=l, weights=None if w is None else w[:n]))
 
-    hsteps = min(args.steps, 500)
-    for k in range(20):
-        forward_from_host(k)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(hsteps):
-        forward_from_host(k)
-    torch.cuda.synchronize()
-    el_host = time.perf_counter() - t0
-    host_lookups = sum(lookups[k % NB] for k in range(hsteps))
+    hsteps = 0 if args.no_pcie else min(args.steps, 500)
+    el_host, host_lookups = 0.0, 0
+    if hsteps:
+        for k in range(20):
+            forward_from_host(k)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(hsteps):
+            forward_from_host(k)
+        torch.cuda.synchronize()
+        el_host = time.perf_counter() - t0
+        host_lookups = sum(lookups[k % NB] for k in range(hsteps))
 
     # ---- kernel-only timing: the lookup launch(es) alone, HIP events on the launch stream
     tbe = module._emb_modules[0]
@@ -587,10 +592,16 @@ def main():
         return info.value.decode().split("; ")
 
     def time_launches(fn):
-        for k in range(min(args.warmup, 200)):
-            fn(k % NB)
+        # The first event is recorded behind the warm-up launches without a
+        # synchronization in between: the GPU is then still busy with them and
+        # the timed launches are already queued when it reaches the event, so
+        # the interval holds the launches back to back and not the few
+        # microseconds the host needs to enqueue the first one on an idle GPU
+        # (which a short run, --steps 20, would otherwise spread over its launches).
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for k in range(max(min(args.warmup, 200), 4)):
+            fn(k % NB)
         e0.record()
         for k in range(args.steps):
             fn(k % NB)
@@ -695,7 +706,7 @@ def main():
         },
     }
     result["host_enqueue_ms_per_step"] = host_ms
-    result["pcie_inclusive"] = {
+    result["pcie_inclusive"] = None if not hsteps else {
         "value": host_lookups / el_host, "unit": "lookups/s", "ms_per_step": el_host / hsteps * 1e3,
         "note": "ids, lengths and weights copied from pinned host memory before every forward; never the headline value",
     }
