@@ -75,6 +75,32 @@ def length_per_key(lengths: torch.Tensor, num_features: int, stride: int) -> Lis
     return out.tolist()
 
 
+def length_per_key_async(lengths: torch.Tensor, num_features: int, stride: int):
+    """``length_per_key`` split in two: the reduction and its copy to pinned host memory are queued on the
+    current stream now, and the returned function waits for that copy alone and yields the Python list.
+    Work queued on the stream between the two (a lookup, say) does not hold the wait up, and is not held up.
+    """
+    _check_int(lengths, "lengths")
+    lengths = lengths.contiguous()
+    out = torch.empty(num_features, dtype=torch.int64, device=lengths.device)
+    _lib.check(
+        _lib.lib().tra_length_per_key(
+            _lib.ptr(lengths), num_features, stride, int(lengths.dtype == torch.int64),
+            _lib.ptr(out), _lib.current_stream(lengths.device),
+        )
+    )
+    host = torch.empty(num_features, dtype=torch.int64, pin_memory=True)
+    host.copy_(out, non_blocking=True)
+    arrived = torch.cuda.Event()
+    arrived.record()
+
+    def finish() -> List[int]:
+        arrived.synchronize()
+        return host.tolist()
+
+    return finish
+
+
 def permute_2D_sparse_data(
     permute: torch.Tensor,
     lengths: torch.Tensor,

@@ -753,11 +753,23 @@ class EmbeddingCollection(EmbeddingCollectionInterface, ModuleNoCopyMixin, _Feat
         offsets = features.offsets()
         lengths = features.lengths().view(len(kjt_keys), -1) if kjt_keys else features.lengths()
         L = indices.numel()
-        # Row ranges of the input keys: one small device-to-host copy.  Asked for
-        # before the lookup is launched, so that the host waits here only for
-        # work that is already queued and then builds the output views while
-        # the lookup runs.
-        offset_per_key = features.offset_per_key()
+        # Row ranges of the input keys: one small device-to-host copy.  Where the
+        # KJT does not carry the per-key counts, their reduction and copy are
+        # queued in front of the lookup and waited for behind its launch: the
+        # host then waits for work that is already queued and builds the output
+        # views while the lookup runs, and the lookup never waits for the host.
+        counts_later = None
+        if (
+            features.length_per_key_or_none() is None
+            and features.offset_per_key_or_none() is None
+            and indices.is_cuda
+            and kjt_keys
+            and L > 0
+            and B > 0
+        ):
+            counts_later = ops.length_per_key_async(features.lengths(), len(kjt_keys), B)
+        else:
+            offset_per_key = features.offset_per_key()
         lookup = torch.empty((L, self._embedding_dim), dtype=self._output_dtype, device=indices.device)
         f0 = 0
         for emb_module, n_feat in zip(self._emb_modules, self._feature_splits):
@@ -769,6 +781,9 @@ class EmbeddingCollection(EmbeddingCollectionInterface, ModuleNoCopyMixin, _Feat
                 out=lookup,
             )
             f0 += n_feat
+        if counts_later is not None:
+            features._length_per_key = counts_later()  # the KJT remembers them, as length_per_key() would
+            offset_per_key = features.offset_per_key()
         if getattr(self, MODULE_ATTR_USE_BATCHING_HINTED_OUTPUT, True):
             lookup = _get_batching_hinted_output(lengths=lengths, output=lookup)
         lengths_rows = torch.unbind(lengths, dim=0) if kjt_keys else ()
