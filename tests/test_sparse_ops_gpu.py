@@ -49,6 +49,11 @@ def test_length_per_key(F, B):
     lengths = rng.integers(0, 41, F * B).astype(np.int32)
     got = ops.length_per_key(torch.from_numpy(lengths).to(DEV), F, B)
     assert got == lengths.reshape(F, B).sum(axis=1).tolist()
+    # the two-step form: queued now, collected after other work has been queued behind it
+    later = ops.length_per_key_async(torch.from_numpy(lengths).to(DEV), F, B)
+    busy = torch.empty(1 << 22, device=DEV).normal_()
+    assert later() == got
+    del busy
 
 
 @pytest.mark.parametrize("T,B,Tp", [(3, 3, 3), (5, 17, 9), (26, 512, 26), (4, 1000, 2), (2, 1, 6)])
