@@ -75,24 +75,40 @@ def length_per_key(lengths: torch.Tensor, num_features: int, stride: int) -> Lis
     return out.tolist()
 
 
+_side_streams: dict = {}  # device index -> a second stream (default priority) for small reads that need not order with the main one
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    s = _side_streams.get(idx)
+    if s is None:
+        s = _side_streams[idx] = torch.cuda.Stream(device=idx)
+    return s
+
+
 def length_per_key_async(lengths: torch.Tensor, num_features: int, stride: int):
-    """``length_per_key`` split in two: the reduction and its copy to pinned host memory are queued on the
-    current stream now, and the returned function waits for that copy alone and yields the Python list.
-    Work queued on the stream between the two (a lookup, say) does not hold the wait up, and is not held up.
-    """
+    """``length_per_key`` split in two: the reduction and its copy to pinned host memory are queued now, on a
+    second stream that waits for what the current stream holds at this moment (whatever produced ``lengths``),
+    and the returned function waits for that copy alone and yields the Python list.  Work queued on the
+    current stream afterwards (a lookup, say) neither waits for the reduction nor holds the host up.
+    ``lengths`` must stay alive until the returned function has been called."""
     _check_int(lengths, "lengths")
     lengths = lengths.contiguous()
-    out = torch.empty(num_features, dtype=torch.int64, device=lengths.device)
-    _lib.check(
-        _lib.lib().tra_length_per_key(
-            _lib.ptr(lengths), num_features, stride, int(lengths.dtype == torch.int64),
-            _lib.ptr(out), _lib.current_stream(lengths.device),
+    dev = lengths.device
+    side = _side_stream(dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        out = torch.empty(num_features, dtype=torch.int64, device=dev)
+        _lib.check(
+            _lib.lib().tra_length_per_key(
+                _lib.ptr(lengths), num_features, stride, int(lengths.dtype == torch.int64),
+                _lib.ptr(out), _lib.current_stream(dev),
+            )
         )
-    )
-    host = torch.empty(num_features, dtype=torch.int64, pin_memory=True)
-    host.copy_(out, non_blocking=True)
-    arrived = torch.cuda.Event()
-    arrived.record()
+        host = torch.empty(num_features, dtype=torch.int64, pin_memory=True)
+        host.copy_(out, non_blocking=True)
+        arrived = torch.cuda.Event()
+        arrived.record(side)
 
     def finish() -> List[int]:
         arrived.synchronize()
