@@ -592,16 +592,10 @@ def main():
         return info.value.decode().split("; ")
 
     def time_launches(fn):
-        # The first event is recorded behind the warm-up launches without a
-        # synchronization in between: the GPU is then still busy with them and
-        # the timed launches are already queued when it reaches the event, so
-        # the interval holds the launches back to back and not the few
-        # microseconds the host needs to enqueue the first one on an idle GPU
-        # (which a short run, --steps 20, would otherwise spread over its launches).
+        for k in range(min(args.warmup, 200)):
+            fn(k % NB)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for k in range(max(min(args.warmup, 200), 4)):
-            fn(k % NB)
         e0.record()
         for k in range(args.steps):
             fn(k % NB)
