@@ -358,6 +358,55 @@ def test_position_weights_inside_the_lookup_kernel(B, max_len, idt, from_offsets
 
 
 @pytest.mark.gpu
+def test_scratch_address_follows_a_replaced_buffer():
+    """The operator remembers the scratch address per call shape.  A larger call
+    replaces the stream's buffer: the addresses remembered for smaller shapes go
+    with it, on the plain route and on the position-weighted one alike."""
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(5)
+    rows, D = 300, 32
+    q = torch.from_numpy(O.quantize_sbhalf(rng.normal(0, 0.1, (rows, D)).astype(np.float32), 8))
+    cfg = EmbeddingBagConfig(name="t", embedding_dim=D, num_embeddings=rows, feature_names=["a", "b"],
+                             data_type=DataType.INT8)
+    pw = PositionWeightedModuleCollection({"a": 9, "b": 9}, dev)
+    with torch.no_grad():
+        for p in pw.position_weights.values():
+            p.copy_(torch.rand_like(p) + 0.5)
+    m = QuantFPEBC([cfg], True, dev, table_name_to_quantized_weights={"t": (q[:, :-4].to(dev), q[:, -4:].to(dev))},
+                   feature_processor=pw)
+    op = m._emb_modules[0]
+
+    def kjt_of(B):
+        lengths = rng.integers(0, 9, 2 * B).astype(np.int32)
+        ids = rng.integers(0, rows, int(lengths.sum())).astype(np.int32)
+        return KeyedJaggedTensor(keys=["a", "b"], values=torch.from_numpy(ids).to(dev),
+                                 lengths=torch.from_numpy(lengths).to(dev))
+
+    def remembered_addresses_are_live():
+        for (_, _, _, stream), address in op._ws_ptr.items():
+            assert address == op._workspace[stream].data_ptr()
+
+    def weighted_from_lengths(kjt):
+        # the weights materialized, the KJT still without offsets: the plain lengths route
+        return KeyedJaggedTensor(keys=kjt.keys(), values=kjt.values(), weights=pw(kjt).weights(),
+                                 lengths=kjt.lengths())
+
+    small, large = kjt_of(48), kjt_of(20000)
+    plain_small = QuantEBC.forward(m, weighted_from_lengths(small)).values().clone()
+    fused_small = m(small).values().clone()                         # position-weighted route, same shape
+    assert torch.equal(plain_small, fused_small)
+    assert op._ws_ptr, "neither route took scratch: the test covers nothing"
+    remembered_addresses_are_live()
+    fused_large = m(large).values().clone()                         # replaces the buffer
+    remembered_addresses_are_live()
+    assert torch.equal(QuantEBC.forward(m, weighted_from_lengths(small)).values(), plain_small)
+    assert torch.equal(m(small).values(), fused_small)
+    remembered_addresses_are_live()
+    assert torch.equal(fused_large, QuantEBC.forward(m, weighted_from_lengths(large)).values())
+    assert torch.equal(fused_large, QuantEBC.forward(m, pw(large)).values())
+
+
+@pytest.mark.gpu
 def test_position_weighted_entry_checks_its_layout():
     """The C entry point validates the host-side layout against the table."""
     dev = torch.device("cuda:0")

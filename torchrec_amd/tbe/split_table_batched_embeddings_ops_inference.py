@@ -419,11 +419,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             ws_ptr = None
             if offsets is None:
                 assert k_total == n_k, "one (start, length) pair per key of the lengths"
-                ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
-                ws = self._workspace.get(stream)
-                if ws is None or ws.numel() < ws_bytes or ws.device != dev:
-                    ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
-                ws_ptr = ws.data_ptr()
+                ws_ptr = self._scratch_address(k_total, B, i64, stream)
             _lib.check(
                 _lib.lib().tra_tbe_forward_position_weighted(
                     self._get_plan(positions), _lib.ptr(self.weights_dev), _lib.ptr(indices),
@@ -449,6 +445,24 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 raise IndexError(f"{bad} embedding indices were out of range")
         return out
 
+    def _scratch_address(self, k_total: int, B: int, i64: int, stream: int) -> int:
+        """Device address of the lengths entry points' scratch for this call shape on this stream
+        (one buffer per stream: calls queued on different streams must not share it).  A shape seen
+        before costs one dictionary lookup."""
+        ws_key = (k_total, B, i64, stream)
+        ws_ptr = self._ws_ptr.get(ws_key)
+        if ws_ptr is None:
+            dev = self.current_device
+            ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
+            ws = self._workspace.get(stream)
+            if ws is None or ws.numel() < ws_bytes or ws.device != dev:
+                ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+                # a larger buffer replaced the stream's old one: forget the addresses handed out from it
+                for k in [k for k in self._ws_ptr if k[3] == stream]:
+                    del self._ws_ptr[k]
+            ws_ptr = self._ws_ptr[ws_key] = ws.data_ptr()
+        return ws_ptr
+
     def _launch_from_lengths(
         self,
         positions: Optional[Tuple[int, ...]],
@@ -465,21 +479,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         """The launch of ``forward(offsets=None, lengths=...)``.  The caller has checked the arguments:
         contiguous device tensors on this operator's GPU, ``lengths`` of the ids' type with ``k_total * B``
         entries, ``psw`` fp32 or None."""
-        dev = self.current_device
-        stream = _lib.current_stream(dev)
-        # The scratch buffer of this call shape on this stream (one per stream: calls queued on
-        # different streams must not share it), found again by one dictionary lookup.
-        ws_key = (k_total, B, i64, stream)
-        ws_ptr = self._ws_ptr.get(ws_key)
-        if ws_ptr is None:
-            ws_bytes = _lib.lib().tra_tbe_forward_lengths_workspace_bytes(k_total, B, i64)
-            ws = self._workspace.get(stream)
-            if ws is None or ws.numel() < ws_bytes or ws.device != dev:
-                ws = self._workspace[stream] = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
-                # a larger buffer replaced the stream's old one: forget the addresses handed out from it
-                for k in [k for k in self._ws_ptr if k[3] == stream]:
-                    del self._ws_ptr[k]
-            ws_ptr = self._ws_ptr[ws_key] = ws.data_ptr()
+        stream = _lib.current_stream(self.current_device)
+        ws_ptr = self._scratch_address(k_total, B, i64, stream)
         global _FORWARD_LENGTHS
         fn = _FORWARD_LENGTHS
         if fn is None:
