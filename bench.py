@@ -42,7 +42,9 @@ def parse_args():
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
     p.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
-    p.add_argument("--batches", type=int, default=8, help="distinct id batches rotated through")
+    p.add_argument("--batches", type=int, default=None,
+                   help="distinct id batches rotated through (default 32 for c2, whose 8-batch cycle half fits the "
+                        "256 MB memory-side cache and then reads 8 %% fast; 8 elsewhere: those cycles are far larger)")
     p.add_argument("--mode", default="eager", choices=["graph", "eager"])
     p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
     p.add_argument("--alt-row-alignment", type=int, default=None,
@@ -357,6 +359,38 @@ def rocprof_summary(root):
             print(f"{len(v):10d} {sum(v) / len(v):20.1f}  {c}  {k}")
 
 
+KERNEL_MIN_LAUNCHES = 200
+KERNEL_MIN_WARMUP = 500
+
+
+def time_kernel_launches(fn, steps, warmup, nb):
+    """Average period of a lookup launch in a queue that stays full: ``fn(batch)``
+    is launched ``max(warmup, 500)`` times untimed, then, with no wait in between,
+    ``max(steps, 200)`` times between two HIP events recorded on the launching
+    stream.  The first event is reached when the last untimed launch ends, the
+    second when the last timed one ends, so the quotient is the steady-state time
+    per launch (its kernel plus the gap to the next one).  The counts have floors
+    because the quantity is a property of the kernel, not of the run's length: a
+    region of 20 launches that opens on a GPU which has idled through set-up reads
+    1 to 2 us more per 24 us launch than the same launches deep inside a long run
+    (the first few hundred launches after an idle stretch are slower), and that
+    start-up belongs to ``ms_per_step``, whose region does open so.
+    Returns (ms per launch, launches timed)."""
+    import torch
+
+    n = max(steps, KERNEL_MIN_LAUNCHES)
+    torch.cuda.synchronize()
+    for k in range(max(warmup, KERNEL_MIN_WARMUP)):
+        fn(k % nb)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for k in range(n):
+        fn(k % nb)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n, n
+
+
 def measure_alt_layout(args, dev, row_alignment, ref_out):
     """The same workload (same seeds: same tables, same ids) stored with another
     row alignment: step time of the module forward, kernel time of its lookup
@@ -403,23 +437,14 @@ def measure_alt_layout(args, dev, row_alignment, ref_out):
                                                wl["B"], wl["T"], v.numel(), int(tbe.pooling_mode), tbe.output_dtype,
                                                _lib.ptr(kout), kout.stride(0), _lib.ptr(ws), stream))
 
-    for k in range(warm):
-        launch(k % NB)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for k in range(steps):
-        launch(k % NB)
-    e1.record()
-    torch.cuda.synchronize()
-    call_ms = e0.elapsed_time(e1) / steps
-    alg = sum(wl["alg_bytes"][k % NB] for k in range(steps)) / steps
+    call_ms, timed_launches = time_kernel_launches(launch, steps, warm, NB)
+    alg = sum(wl["alg_bytes"][k % NB] for k in range(timed_launches)) / timed_launches
     lookups = sum(batches[k % NB][0].numel() for k in range(steps))
     return {
         "row_alignment": row_alignment,
         "store_GB": wl["store_bytes"] / 1e9,
         "value": lookups / el, "unit": "lookups/s", "ms_per_step": el / steps * 1e3,
-        "lookup_call_ms": call_ms, "launches_per_call": launches,
+        "lookup_call_ms": call_ms, "launches_timed": timed_launches, "launches_per_call": launches,
         "achieved": alg / (call_ms * 1e-3) / 1e9, "frac": alg / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "outputs_equal_default_layout": same,
         "note": "same tables and ids, rows padded to the given alignment (QuantEmbeddingBagCollection(row_alignment=...)); "
@@ -435,6 +460,8 @@ def main():
         return
     if args.row_alignment is None:
         args.row_alignment = 4 if args.config == "c5" else 16
+    if args.batches is None:
+        args.batches = 32 if args.config == "c2" else 8
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
         sys.exit(2)
@@ -519,8 +546,9 @@ def main():
     # host-side cost of a step: the same loop without waiting for the GPU
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    run("eager", min(args.steps, 500))
-    host_ms = (time.perf_counter() - t0) / min(args.steps, 500) * 1e3
+    host_steps = min(max(args.steps, 200), 500)
+    run("eager", host_steps)
+    host_ms = (time.perf_counter() - t0) / host_steps * 1e3
     torch.cuda.synchronize()
 
     # ---- the same step fed from pinned host memory (ids, lengths, weights cross PCIe every step)
@@ -592,16 +620,7 @@ def main():
         return info.value.decode().split("; ")
 
     def time_launches(fn):
-        for k in range(min(args.warmup, 200)):
-            fn(k % NB)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for k in range(args.steps):
-            fn(k % NB)
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / args.steps
+        return time_kernel_launches(fn, args.steps, args.warmup, NB)
 
     # The module's forward hands a KJT built from lengths to the operator's
     # lengths entry point; when that derives the offsets inside the lookup
@@ -610,9 +629,9 @@ def main():
     fused = any(x.endswith("from_lengths") for x in launches)
     if not fused:
         launches = launch_info(0)
-    alg = sum(wl["alg_bytes"][k % args.batches] for k in range(args.steps)) / args.steps
     step_launch = launch_lengths if fused else launch_offsets
-    kernel_ms = time_launches(step_launch)
+    kernel_ms, timed_launches = time_launches(step_launch)
+    alg = sum(wl["alg_bytes"][k % args.batches] for k in range(timed_launches)) / timed_launches
     achieved = alg / (kernel_ms * 1e-3) / 1e9
     # spread of single launches: one event pair per launch (includes the launch gap)
     singles = []
@@ -626,7 +645,7 @@ def main():
     single_us = sorted(x.elapsed_time(y) * 1e3 for x, y in singles)
     offsets_entry = None
     if fused:
-        ms = time_launches(launch_offsets)
+        ms, _ = time_launches(launch_offsets)
         offsets_entry = {
             "kernel_ms": ms, "achieved": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "launches_per_call": launch_info(0),
@@ -692,6 +711,10 @@ def main():
             "kernel": launches[0].split(" ")[0],
             "launches_per_call": launches,
             "kernel_ms": kernel_ms,
+            "kernel_launches_timed": timed_launches,
+            "kernel_timing": "HIP events around the timed launches, queued behind the untimed ones with no wait in "
+                             "between (steady state); at least 500 untimed and 200 timed launches whatever --warmup "
+                             "and --steps say",
             "algorithmic_bytes_per_launch": alg,
             "kernel_lookups_per_s": (sum(lookups) / NB) / (kernel_ms * 1e-3),
             "single_launch_us_p50": single_us[len(single_us) // 2],
