@@ -895,6 +895,107 @@ def test_random_plans(tuning, seed):
     assert tbe.out_of_range_count() == 0, tag
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_natural_key_order(tuning, seed):
+    """Seeded random operators whose features sit at consecutive key positions
+    (what a collection with one feature per table launches), window kernel
+    forced with windows of 64 - 300 bags: the lengths entry (up to 256 bags the
+    window is staged by one wave while the others sum the prefix) and the
+    offsets entry against the oracle, bit for bit."""
+    rng = np.random.default_rng(50000 + seed)
+    nt = int(rng.integers(1, 9))
+    pooling = [O.SUM, O.MEAN][int(rng.integers(0, 2))]
+    dims_pool = [16, 32, 64, 128, 256]
+    same = bool(rng.integers(0, 2))
+    dt0 = [O.INT8, O.INT4, O.INT2, O.FP16][int(rng.integers(0, 4))]
+    d0 = dims_pool[int(rng.integers(0, 5))]
+    specs = []
+    for _ in range(nt):
+        dt = dt0 if same else [O.INT8, O.INT4, O.INT2, O.FP16, O.FP32][int(rng.integers(0, 5))]
+        dim = d0 if same else dims_pool[int(rng.integers(0, 5))]
+        specs.append((dt, int(rng.choice([3, 500, 3000])), dim))
+    ftm = list(range(nt))
+    out_dtype = [O.FP32, O.FP16][int(rng.integers(0, 2))]
+    ra = int(rng.choice([4, 16, 64]))
+    idt = [np.int32, np.int64][int(rng.integers(0, 2))]
+    B = int(rng.choice([3, 64, 100, 257, 700]))
+    max_len = int(rng.choice([1, 5, 40, 200, 400]))
+    if max_len >= 200:
+        B = min(B, 64)
+    weighted = bool(rng.integers(0, 2))
+    window = int(rng.choice([64, 100, 208, 256, 300]))
+    tuning(balanced=1)
+    tuning(window=window)
+    tbe, store = build(rng, specs, ftm, pooling, out_dtype, ra)
+    lengths, offsets, ids = make_bags(rng, [s[1] for s in specs], B, max_len, idt,
+                                      empty_frac=float(rng.choice([0.0, 0.1, 0.5])))
+    if len(ids):
+        ids[rng.random(len(ids)) < 0.03] = -1
+    psw = rng.uniform(-2, 2, len(ids)).astype(np.float32) if weighted else None
+    want = O.tbe_forward(store, ftm, B, ids, offsets, psw, pooling, out_dtype)
+    tag = (seed, specs, pooling, out_dtype, ra, idt.__name__, B, max_len, weighted, window)
+    assert bits_equal(_from_lengths(tbe, ids, lengths, psw, B), want) == 0, tag
+    got = tbe(torch.from_numpy(ids).to(DEV), torch.from_numpy(offsets).to(DEV),
+              None if psw is None else torch.from_numpy(psw).to(DEV)).cpu().numpy()
+    assert bits_equal(got, want) == 0, tag
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_position_weights(tuning, seed):
+    """Seeded random operators with the position weights looked up inside the
+    lookup kernel (static and window kernel, offsets and lengths entry, keys with
+    0, 1 or many weights, bags longer than their weight vector): same bits as
+    the oracle fed with the weights materialized per id."""
+    rng = np.random.default_rng(70000 + seed)
+    nt = int(rng.integers(1, 7))
+    pooling = [O.SUM, O.MEAN][int(rng.integers(0, 2))]
+    dims_pool = [16, 32, 64, 128, 256]
+    specs = [([O.INT8, O.INT4, O.INT2, O.FP16, O.FP32][int(rng.integers(0, 5))], int(rng.choice([3, 500, 3000])),
+              dims_pool[int(rng.integers(0, 5))]) for _ in range(nt)]
+    ftm = list(range(nt)) + [int(x) for x in rng.integers(0, nt, int(rng.integers(0, 3)))]
+    if rng.integers(0, 2):
+        rng.shuffle(ftm)
+    nk = len(ftm)
+    out_dtype = [O.FP32, O.FP16][int(rng.integers(0, 2))]
+    ra = int(rng.choice([4, 16, 64]))
+    idt = [np.int32, np.int64][int(rng.integers(0, 2))]
+    B = int(rng.choice([3, 64, 257, 700]))
+    max_len = int(rng.choice([1, 5, 40, 200]))
+    if max_len >= 200:
+        B = min(B, 64)
+    route = ["static", "window"][int(rng.integers(0, 2))]
+    window = int(rng.choice([64, 100, 208, 256, 300]))
+    from_lengths = bool(rng.integers(0, 2))
+    key_len = [int(rng.choice([0, 1, 7, 30, 250])) for _ in range(nk)]
+    key_start, tot = [], 0
+    for n_ in key_len:
+        key_start.append(tot)
+        tot += n_
+    table = rng.uniform(-1.5, 1.5, max(tot, 1)).astype(np.float32)
+    tuning(balanced=1 if route == "window" else 0)
+    if route == "window":
+        tuning(window=window)
+    tbe, store = build(rng, specs, ftm, pooling, out_dtype, ra)
+    lengths, offsets, ids = make_bags(rng, [specs[t][1] for t in ftm], B, max_len, idt,
+                                      empty_frac=float(rng.choice([0.0, 0.1, 0.5])))
+    psw = np.ones(len(ids), dtype=np.float32)
+    for k in range(nk):
+        if key_len[k] == 0:
+            continue  # a key without weights: every id weighs 1
+        for b in range(B):
+            s, e = int(offsets[k * B + b]), int(offsets[k * B + b + 1])
+            psw[s:e] = table[key_start[k] + np.minimum(np.arange(e - s), key_len[k] - 1)]
+    want = O.tbe_forward(store, ftm, B, ids, offsets, psw, pooling, out_dtype)
+    pw = (torch.from_numpy(table).to(DEV), key_start, key_len)
+    ti = torch.from_numpy(ids).to(DEV)
+    if from_lengths:
+        got = tbe(ti, None, None, lengths=torch.from_numpy(lengths).to(DEV), batch_size=B, position_weights=pw)
+    else:
+        got = tbe(ti, torch.from_numpy(offsets).to(DEV), None, position_weights=pw)
+    tag = (seed, specs, ftm, pooling, out_dtype, ra, idt.__name__, B, max_len, route, window, from_lengths, key_len)
+    assert bits_equal(got.cpu().numpy(), want) == 0, tag
+
+
 def test_table_beyond_2_31_rows(tuning):
     """A table with more than 2^31 rows (fp32, dim 1: 8.6 GB): int64 ids beyond 2^31 address the
     right rows; int32 ids see every non-negative id as in range; ids >= rows are skipped and counted."""
