@@ -77,6 +77,58 @@ def test_permute_2d(T, B, Tp, idt, vdt, weighted):
         assert gw is None
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("weighted", [False, True])
+def test_permute_2d_selecting_only_empty_features(weighted):
+    """A permutation that picks nothing but features without ids, out of an input
+    that has ids (and weights) elsewhere: empty outputs, no call with null outputs."""
+    lengths = np.array([[2, 1, 3], [0, 0, 0], [1, 1, 1], [0, 0, 0]], dtype=np.int64)
+    total = int(lengths.sum())
+    values = np.arange(total, dtype=np.int64)
+    weights = np.linspace(0, 1, total).astype(np.float32) if weighted else None
+    perm = np.array([3, 1, 1], dtype=np.int32)
+    gl, gv, gw = ops.permute_2D_sparse_data(
+        torch.from_numpy(perm).to(DEV), torch.from_numpy(lengths).to(DEV), torch.from_numpy(values).to(DEV),
+        None if weights is None else torch.from_numpy(weights).to(DEV))
+    assert gl.shape == (3, 3) and int(gl.sum()) == 0
+    assert gv.numel() == 0 and gv.dtype == torch.int64
+    assert (gw is None) if not weighted else (gw.numel() == 0 and gw.dtype == torch.float32)
+    # through the KJT: the permuted tensor is usable
+    from torchrec_amd import KeyedJaggedTensor
+    kjt = KeyedJaggedTensor(keys=["a", "b", "c", "d"], values=torch.from_numpy(values).to(DEV),
+                            lengths=torch.from_numpy(lengths.reshape(-1)).to(DEV),
+                            weights=None if weights is None else torch.from_numpy(weights).to(DEV))
+    p = kjt.permute([3, 1])
+    assert p.keys() == ["d", "b"] and p.values().numel() == 0 and p.lengths().tolist() == [0] * 6
+
+
+@pytest.mark.gpu
+def test_ops_with_bags_but_no_ids_to_write():
+    """Operators whose output is empty while their input is not (or whose bags
+    hold no ids at all) return empty tensors; they pass no null output on."""
+    F, B, W = 3, 4, 2
+    zero = torch.zeros(F * B, dtype=torch.int64, device=DEV)
+    offsets0 = torch.zeros(F * B + 1, dtype=torch.int64, device=DEV)
+    # position weights of bags without ids
+    out = ops.position_weights(offsets0, F, B, torch.zeros(F, dtype=torch.int32, device=DEV),
+                               torch.full((F,), 5, dtype=torch.int32, device=DEV), torch.ones(15, device=DEV), 0)
+    assert out.numel() == 0 and out.dtype == torch.float32
+    assert ops.offsets_range(offsets0[:-1], 0).numel() == 0
+    # bucketize: no ids at all
+    empty = torch.zeros(0, dtype=torch.int64, device=DEV)
+    bs = torch.full((F,), 10, dtype=torch.int64, device=DEV)
+    nl, ni, nw, _, nu = ops.block_bucketize_sparse_features(zero, empty, False, True, bs, W, torch.zeros(0, device=DEV))
+    assert int(nl.sum()) == 0 and ni.numel() == 0 and nw.numel() == 0 and nu.numel() == 0
+    # bucketize: ids and weights present, every id beyond the last bucket (dropped)
+    lengths = torch.ones(F * B, dtype=torch.int64, device=DEV)
+    ids = torch.full((F * B,), 10 * W + 3, dtype=torch.int64, device=DEV)
+    nl, ni, nw, _, _ = ops.block_bucketize_sparse_features(lengths, ids, False, False, bs, W, torch.rand(F * B, device=DEV))
+    want = O.bucketize(lengths.cpu().numpy(), ids.cpu().numpy(), bs.cpu().numpy(), W,
+                       np.ones(F * B, dtype=np.float32), False)
+    assert nl.cpu().numpy().tolist() == want[0].tolist() and int(nl.sum()) == 0
+    assert ni.numel() == len(want[1]) == 0 and nw.numel() == 0
+
+
 @pytest.mark.parametrize("F,B,W", [(1, 1, 1), (2, 3, 2), (4, 15, 5), (15, 15, 129), (3, 200, 8)])
 @pytest.mark.parametrize("idt", [np.int32, np.int64])
 @pytest.mark.parametrize("keep", [False, True])

@@ -170,13 +170,14 @@ def permute_2D_sparse_data(
         if weights.dtype != torch.float32:
             raise TypeError(f"weights must be float32, got {weights.dtype}")
         out_weights = torch.empty(permuted_lengths_sum, dtype=torch.float32, device=dev)
-    _lib.check(
-        l.tra_permute_2d_data(
-            _lib.ptr(permute), Tp, B, _lib.ptr(in_offsets), _lib.ptr(out_offsets), is64,
-            _lib.ptr(values), values.element_size(), _lib.ptr(weights), _lib.ptr(out_values),
-            _lib.ptr(out_weights), stream,
+    if permuted_lengths_sum > 0:  # (nothing to move otherwise, and empty outputs have no address to pass)
+        _lib.check(
+            l.tra_permute_2d_data(
+                _lib.ptr(permute), Tp, B, _lib.ptr(in_offsets), _lib.ptr(out_offsets), is64,
+                _lib.ptr(values), values.element_size(), _lib.ptr(weights), _lib.ptr(out_values),
+                _lib.ptr(out_weights), stream,
+            )
         )
-    )
     return out_lengths, out_values, out_weights
 
 
@@ -240,7 +241,9 @@ def block_bucketize_sparse_features(
     cursor = torch.empty(ws_bytes // 8, dtype=torch.int64, device=dev) if ws_bytes else None
     _lib.check(
         l.tra_bucketize_scatter(
-            _lib.ptr(offsets), _lib.ptr(indices), is64, _lib.ptr(weights), _lib.ptr(bs), F, B, W,
+            # (no id kept, e.g. all beyond the last bucket: no weight is moved, and the empty
+            # output has no address to pass)
+            _lib.ptr(offsets), _lib.ptr(indices), is64, _lib.ptr(weights if total > 0 else None), _lib.ptr(bs), F, B, W,
             int(keep_orig_idx), _lib.ptr(new_offsets), _lib.ptr(cursor), _lib.ptr(new_indices),
             _lib.ptr(new_weights), _lib.ptr(unbucketize), stream,
         )
@@ -321,6 +324,8 @@ def position_weights(
     assert offsets.numel() >= num_keys * batch_size + 1
     assert key_start.dtype == torch.int32 and key_len.dtype == torch.int32 and table.dtype == torch.float32
     out = torch.empty(num_values, dtype=torch.float32, device=offsets.device)
+    if num_values == 0:  # (bags without ids: nothing to weigh, and an empty output has no address to pass)
+        return out
     _lib.check(
         _lib.lib().tra_position_weights(
             _lib.ptr(offsets), int(offsets.dtype == torch.int64), num_keys, batch_size, _lib.ptr(key_start),
