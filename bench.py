@@ -61,6 +61,10 @@ def parse_args():
     p.add_argument("--rocprof-summary", metavar="DIR", default=None,
                    help="no benchmark: summarize rocprofv3 CSV output under DIR (kernel_stats / counter_collection) "
                         "for this library's kernels and exit")
+    p.add_argument("--id-permutation", default="fixed", choices=["fixed", "per-batch"],
+                   help="c2: rank -> id through one seeded permutation per table shared by all batches (the named "
+                        "workload), or through a new permutation for every batch (cold head: no row is hot in two "
+                        "batches; a lower bound, not the named workload)")
     p.add_argument("--batch-size", type=int, default=None, help="override the workload's batch size (tuning only; result is then not the named workload)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink table rows (debug only; result is then invalid)")
     return p.parse_args()
@@ -69,20 +73,40 @@ def parse_args():
 # --------------------------------------------------------------------------
 # workloads
 # --------------------------------------------------------------------------
-def zipf_ids(n, rows, alpha, gen, device):
-    """n ids with rank ~ truncated Zipf(alpha) on [1, rows], rank -> id through a seeded permutation."""
-    import torch
+class ZipfTable:
+    """Id source of one table: rank ~ truncated Zipf(alpha) on [1, rows], id = perm[rank - 1].
 
-    if n == 0:
-        return torch.zeros(0, dtype=torch.int64, device=device)
-    w = torch.arange(1, rows + 1, dtype=torch.float64, device=device).pow_(-alpha)
-    cdf = torch.cumsum(w, 0)
-    cdf /= cdf[-1].clone()
-    u = torch.rand(n, dtype=torch.float64, device=device, generator=gen)
-    rank = torch.searchsorted(cdf, u).clamp_(max=rows - 1)
-    del w, cdf, u
-    perm = torch.randperm(rows, device=device, generator=gen)
-    return perm[rank]
+    The permutation is drawn ONCE per table, from a generator seeded by (workload
+    seed, table), and every batch draws its ids through it: the hot rows of a
+    table are the same rows in every batch, as they are for a model in service.
+    Only the ranks differ from batch to batch."""
+
+    def __init__(self, rows, alpha, seed, table, device):
+        import torch
+
+        g = torch.Generator(device=device)
+        g.manual_seed(seed * 1_000_003 + table)
+        self.rows = rows
+        w = torch.arange(1, rows + 1, dtype=torch.float64, device=device).pow_(-alpha)
+        cdf = torch.cumsum(w, 0)
+        cdf /= cdf[-1].clone()
+        self.cdf = cdf
+        self.perm = torch.randperm(rows, device=device, generator=g).to(torch.int32)
+
+    def draw(self, n, gen, fresh_permutation=False):
+        import torch
+
+        if fresh_permutation:  # the rows that are hot change with every batch (no reuse from batch to batch)
+            self.perm = torch.randperm(self.rows, device=self.perm.device, generator=gen).to(torch.int32)
+        if n == 0:
+            return torch.zeros(0, dtype=torch.int64, device=self.perm.device)
+        u = torch.rand(n, dtype=torch.float64, device=self.perm.device, generator=gen)
+        rank = torch.searchsorted(self.cdf, u).clamp_(max=self.rows - 1)
+        return self.perm[rank].long()
+
+    def hottest(self, k):
+        """The ids of ranks 1..k."""
+        return self.perm[:k].long()
 
 
 def build_workload(args, dev):
@@ -102,12 +126,13 @@ def build_workload(args, dev):
     DT = {"int8": DataType.INT8, "int4": DataType.INT4, "int2": DataType.INT2, "fp16": DataType.FP16}
 
     weighted, pooled, out_dtype, pooling = False, True, torch.half, PoolingType.SUM
+    zipf = None
     if cfg == "c1":
         T, B = 8, 512
         rows = [100_000] * T
         dims, dts = [64] * T, ["int8"] * T
         lens = lambda: np.full(T * B, 20, dtype=np.int64)
-        id_fn = lambda n, r: torch.randint(0, r, (n,), device=dev, generator=gen)
+        id_fn = lambda n, r, t: torch.randint(0, r, (n,), device=dev, generator=gen)
         desc = "c1: QEBC 8 tables x 100k x 64 int8, B512, L=20, SUM, fp16 out, uniform ids"
     elif cfg == "c2":
         T, B = 26, 2048
@@ -119,15 +144,18 @@ def build_workload(args, dev):
             l[rng.random(T * B) < 0.05] = 0
             return l
 
-        id_fn = lambda n, r: zipf_ids(n, r, 1.05, gen, dev)
-        desc = "c2: QEBC 26 tables rows logU[1e3,4e7] x 128 int4, B2048, len U[1,40] 5% empty, Zipf(1.05), SUM, fp16 out"
+        zipf = [ZipfTable(rows[t], 1.05, seed, t, dev) for t in range(T)]
+        fresh = getattr(args, "id_permutation", "fixed") == "per-batch"
+        id_fn = lambda n, r, t: zipf[t].draw(n, gen, fresh)
+        desc = ("c2: QEBC 26 tables rows logU[1e3,4e7] x 128 int4, B2048, len U[1,40] 5% empty, Zipf(1.05) over one "
+                "seeded permutation per table (the same in every batch), SUM, fp16 out")
     elif cfg == "c3":
         T, B = 64, 4096
         rows = [max(1000, int(round(math.exp(x) * args.scale))) for x in rng.uniform(math.log(1e5), math.log(1e7), T)]
         dims = [[32, 64, 128, 256][t % 4] for t in range(T)]
         dts = [["int8", "int4", "int2", "fp16"][(t // 4) % 4] for t in range(T)]
         lens = lambda: rng.poisson(30, T * B)
-        id_fn = lambda n, r: torch.randint(0, r, (n,), device=dev, generator=gen)
+        id_fn = lambda n, r, t: torch.randint(0, r, (n,), device=dev, generator=gen)
         weighted, out_dtype = True, torch.float
         desc = "c3: QEBC 64 tables mixed D{32..256} x {int8,int4,int2,fp16}, B4096, Poisson(30), weighted SUM, fp32 out"
     elif cfg == "c4":
@@ -135,7 +163,7 @@ def build_workload(args, dev):
         rows = [max(1000, int(1_000_000 * args.scale))] * T
         dims, dts = [128] * T, ["int8"] * T
         lens = lambda: rng.integers(0, 257, T * B)
-        id_fn = lambda n, r: torch.randint(0, r, (n,), device=dev, generator=gen)
+        id_fn = lambda n, r, t: torch.randint(0, r, (n,), device=dev, generator=gen)
         pooled = False
         desc = "c4: QEC 16 tables x 1e6 x 128 int8, B1024, len U[0,256], uniform ids, jagged fp16 out"
     else:
@@ -213,12 +241,19 @@ def build_workload(args, dev):
                 vals.append((rank * mul + 12345 * (t + 1)) % N)
             values = torch.cat(vals)
         else:
-            values = torch.cat([id_fn(int(per[t]), rows[t]) for t in range(T)])
+            values = torch.cat([id_fn(int(per[t]), rows[t], t) for t in range(T)])
         values = values.to(torch.int32)
         lengths = torch.from_numpy(l).to(torch.int32).to(dev)
         w = torch.rand(values.numel(), device=dev, generator=gen) if weighted else None
         batches.append((values, lengths, w))
     torch.cuda.synchronize(dev)
+    hot_ids = None
+    if zipf is not None:
+        hot_ids = [z.hottest(min(16, z.rows)) for z in zipf]
+        if fresh:
+            desc = desc.replace("one seeded permutation per table (the same in every batch)",
+                                "a NEW permutation per table for every batch (cold head)")
+        del zipf, id_fn
 
     # algorithmic bytes per call: unpadded rows + ids + weights + offsets + output
     def alg_bytes(values, lengths):
@@ -234,7 +269,7 @@ def build_workload(args, dev):
 
     return dict(
         module=module, batches=batches, keys=[f"f{t}" for t in range(T)], T=T, B=B, rows=rows, dims=dims, dts=dts,
-        weighted=weighted, pooled=pooled, out_dtype=out_dtype, desc=desc,
+        weighted=weighted, pooled=pooled, out_dtype=out_dtype, desc=desc, hot_ids=hot_ids,
         alg_bytes=[alg_bytes(v, l) for v, l, _ in batches],
         store_bytes=sum(m.weights_size for m in module._emb_modules),
     )
@@ -696,6 +731,8 @@ def main():
             "workload": wl["desc"],
             "step": f"QuantEmbeddingBagCollection.forward(KJT) ({args.mode}), {NB} rotating batches",
             "row_alignment": args.row_alignment,
+            "id_permutation": ("fixed per table" if args.id_permutation == "fixed" else "new per batch (cold head)")
+                              if args.config == "c2" else None,
             "rows_total": int(sum(wl["rows"])),
             "store_GB": wl["store_bytes"] / 1e9,
             "lookups_per_step": sum(lookups) / NB,

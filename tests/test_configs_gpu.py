@@ -131,13 +131,25 @@ def test_config2_full_size_zipf_log_uniform_rows():
     B 2048, lengths U[1,40] with 5 % empty, Zipf(1.05) ids through a permutation."""
     if _free_bytes() < 12e9:
         pytest.skip("needs 12 GB of free device memory")
-    wl = _workload("c2")
+    wl = _workload("c2", batches=2)
     assert min(wl["rows"]) < 5_000 and max(wl["rows"]) > 10_000_000  # the log-uniform spread is there
     out = _forward(wl).values()
     v, l, w = wl["batches"][0]
     # Zipf: a handful of rows take a large share of the lookups
     seg = v[: int(l[:wl["B"]].sum())]
     assert torch.bincount(seg.long()).max().item() > 20
+    # one permutation per table, shared by the batches: the hottest row of every table is the
+    # same row in both batches (and is the rank-1 row of the generator), the ids are not
+    B = wl["B"]
+    big = max(range(wl["T"]), key=lambda t: wl["rows"][t])
+    for t in (0, big, wl["T"] - 1):
+        top = []
+        for vb, lb, _ in wl["batches"]:
+            ends = torch.cumsum(lb.view(wl["T"], B).sum(dim=1), 0)
+            seg_t = vb[int(ends[t - 1]) if t else 0: int(ends[t])].long()
+            top.append(int(torch.bincount(seg_t).argmax()))
+        assert top[0] == top[1] == int(wl["hot_ids"][t][0]), (t, top)
+    assert not torch.equal(wl["batches"][0][0][:1000], wl["batches"][1][0][:1000])
     samples = np.arange(0, wl["B"], 16)  # 128 samples x 26 features
     want = _oracle_on_samples(wl, v, l, w, samples, O.SUM, O.FP16)
     assert bits_equal(np.ascontiguousarray(out[torch.from_numpy(samples).to(DEV)].cpu().numpy()), want) == 0
