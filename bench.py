@@ -47,9 +47,12 @@ def parse_args():
                         "256 MB memory-side cache and then reads 8 %% fast; 8 elsewhere: those cycles are far larger)")
     p.add_argument("--mode", default="eager", choices=["graph", "eager"])
     p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
-    p.add_argument("--alt-row-alignment", type=int, default=None,
-                   help="also measure the same workload with this row alignment (default: 64 for c2, i.e. one "
-                        "128-byte line per row; 0 = skip)")
+    p.add_argument("--row-padding", default=None, choices=["line", "none"],
+                   help="distance between rows in the packed store: 'line' = rows of at most 128 bytes at the next "
+                        "power-of-two stride, so that none straddles a 128-byte line (the operator's default while the "
+                        "padded store fits its budget); 'none' = at their width, the reference's layout")
+    p.add_argument("--no-alt-layout", action="store_true",
+                   help="c2 also measures the same workload with the other row padding; this skips it")
     p.add_argument("--request-streams", type=int, default=3,
                    help="also time the same steps dealt round-robin to this many HIP streams (independent "
                         "requests in flight); 0 or 1 = skip")
@@ -178,6 +181,10 @@ def build_workload(args, dev):
     if getattr(args, "batch_size", None):
         B = args.batch_size
         desc += f" [batch size overridden to {B}]"
+    from torchrec_amd import tbe as _tbe
+    # (c5 is by definition the 68-byte stride: its shortened test shapes must not be padded either)
+    previous_padding = _tbe.set_default_row_padding(
+        getattr(args, "row_padding", None) or ("none" if cfg == "c5" else _tbe.get_default_row_padding()))
     if pooled:
         tables = [
             EmbeddingBagConfig(name=f"t{t}", embedding_dim=dims[t], num_embeddings=rows[t], feature_names=[f"f{t}"],
@@ -192,6 +199,7 @@ def build_workload(args, dev):
             for t in range(T)
         ]
         module = QuantEC(tables, dev, output_dtype=out_dtype, row_alignment=args.row_alignment)
+    _tbe.set_default_row_padding(previous_padding)
 
     # Fill the packed store: fp32 N(0, 0.1) rows quantized on the GPU, chunk by chunk,
     # straight into their header-first rows (c5: synthetic packed bytes, no float master).
@@ -202,7 +210,7 @@ def build_workload(args, dev):
         for t, name in enumerate(tbe.embedding_names):
             gt = int(name[1:])
             view = tbe._rows_view(t)
-            r, rb = tbe.rows[t], tbe.row_bytes[t]
+            r, rb = tbe.rows[t], tbe.row_stride[t]  # distance between rows in the packed store
             step = max(1, (1 << 27) // dims[gt])
             for r0 in range(0, r, step):
                 n = min(step, r - r0)
@@ -307,7 +315,7 @@ def cpu_baseline(wl, out_gpu, seconds):
             tbe.weights_dev.cpu().numpy(),
             np.asarray(tbe.weights_physical_offsets, dtype=np.int64), np.asarray(tbe.rows, dtype=np.int64),
             np.asarray(tbe.dims, dtype=np.int32), np.asarray([code[str(x)] for x in tbe.weight_tys], dtype=np.int32),
-            np.asarray(tbe.row_bytes, dtype=np.int32),
+            np.asarray(tbe.row_stride, dtype=np.int32),
         )
         where = f"whole {tbe.weights_size / 1e9:.2f} GB store in host memory"
     else:
@@ -426,16 +434,16 @@ def time_kernel_launches(fn, steps, warmup, nb):
     return e0.elapsed_time(e1) / n, n
 
 
-def measure_alt_layout(args, dev, row_alignment, ref_out):
-    """The same workload (same seeds: same tables, same ids) stored with another
-    row alignment: step time of the module forward, kernel time of its lookup
-    launch, and whether the outputs equal those of the default layout."""
+def measure_alt_layout(args, dev, row_padding, ref_out):
+    """The same workload (same seeds: same tables, same ids) stored with the other
+    row padding: step time of the module forward, kernel time of its lookup
+    launch, and whether the outputs equal those of the headline layout."""
     import argparse as _ap
     import torch
     from torchrec_amd import _lib, KeyedJaggedTensor
 
     alt = _ap.Namespace(**vars(args))
-    alt.row_alignment = row_alignment
+    alt.row_padding = row_padding
     wl = build_workload(alt, dev)
     module, batches, keys = wl["module"], wl["batches"], wl["keys"]
     NB = len(batches)
@@ -476,14 +484,16 @@ def measure_alt_layout(args, dev, row_alignment, ref_out):
     alg = sum(wl["alg_bytes"][k % NB] for k in range(timed_launches)) / timed_launches
     lookups = sum(batches[k % NB][0].numel() for k in range(steps))
     return {
-        "row_alignment": row_alignment,
+        "row_padding": row_padding,
+        "row_stride_bytes": sorted(set(wl["module"]._emb_modules[0].row_stride)),
         "store_GB": wl["store_bytes"] / 1e9,
         "value": lookups / el, "unit": "lookups/s", "ms_per_step": el / steps * 1e3,
         "lookup_call_ms": call_ms, "launches_timed": timed_launches, "launches_per_call": launches,
         "achieved": alg / (call_ms * 1e-3) / 1e9, "frac": alg / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "outputs_equal_default_layout": same,
-        "note": "same tables and ids, rows padded to the given alignment (QuantEmbeddingBagCollection(row_alignment=...)); "
-                "algorithmic bytes unchanged (unpadded rows); lookup_call_ms covers the whole lookup call "
+        "outputs_equal_headline_layout": same,
+        "note": "same tables and ids, rows stored with the other row padding ('none' = rows at their width, the "
+                "reference's layout; 'line' = power-of-two stride, no row straddles a 128-byte line); algorithmic "
+                "bytes unchanged (unpadded rows); lookup_call_ms covers the whole lookup call "
                 "(tra_tbe_forward_lengths), scan kernels included when it is not fused",
     }
 
@@ -573,6 +583,7 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
+    tbe0 = module._emb_modules[0]
     lookups = [b[0].numel() for b in batches]
     total_lookups = sum(lookups[k % NB] for k in range(args.steps))
     el = timed(args.mode, args.steps, args.warmup)
@@ -731,6 +742,9 @@ def main():
             "workload": wl["desc"],
             "step": f"QuantEmbeddingBagCollection.forward(KJT) ({args.mode}), {NB} rotating batches",
             "row_alignment": args.row_alignment,
+            "row_padding": tbe0.row_padding,
+            "row_bytes": sorted(set(tbe0.row_bytes)),
+            "row_stride_bytes": sorted(set(tbe0.row_stride)),
             "id_permutation": ("fixed per table" if args.id_permutation == "fixed" else "new per batch (cold head)")
                               if args.config == "c2" else None,
             "rows_total": int(sum(wl["rows"])),
@@ -803,12 +817,10 @@ def main():
     if other:
         result["eager_value"] = total_lookups / el_other
         result["eager_ms_per_step"] = el_other / args.steps * 1e3
-    alt_ra = args.alt_row_alignment
-    if alt_ra is None:
-        alt_ra = 64 if args.config == "c2" else 0
-    if alt_ra and alt_ra != args.row_alignment and wl["pooled"]:
-        print(f"[bench] the same workload with row_alignment={alt_ra} ...", file=sys.stderr, flush=True)
-        result["alt_layout"] = measure_alt_layout(args, dev, alt_ra, out_tensor(outs[0]))
+    if args.config == "c2" and not args.no_alt_layout and wl["pooled"]:
+        other_padding = "none" if tbe0.row_stride != tbe0.row_bytes else "line"
+        print(f"[bench] the same workload with row padding '{other_padding}' ...", file=sys.stderr, flush=True)
+        result["alt_layout"] = measure_alt_layout(args, dev, other_padding, out_tensor(outs[0]))
     if not args.no_cpu_baseline:
         print("[bench] timing the CPU baseline ...", file=sys.stderr, flush=True)
         result["cpu_baseline"] = cpu_baseline(wl, out_tensor(outs[0]), args.cpu_seconds)

@@ -89,7 +89,7 @@ def _oracle_on_samples(wl, values, lengths, weights, samples, pooling, out_dtype
         base += rows.size + pad
     store = O.Store(np.concatenate(pieces), np.asarray(t_off, np.int64), np.asarray(t_rows, np.int64),
                     np.asarray(tbe.dims, np.int32), np.asarray([CODE[str(x)] for x in tbe.weight_tys], np.int32),
-                    np.asarray(tbe.row_bytes, np.int32))
+                    np.asarray(tbe.row_bytes, np.int32))  # (rows were gathered at their width)
     return O.tbe_forward(store, list(range(T)), Bs, ids.astype(np.int32), sub_off, w, pooling, out_dtype)
 
 

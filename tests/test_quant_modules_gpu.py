@@ -32,7 +32,7 @@ def oracle_store_of(tbe):
         np.asarray(tbe.rows, dtype=np.int64),
         np.asarray(tbe.dims, dtype=np.int32),
         np.asarray([OCODE[str(t)] for t in tbe.weight_tys], dtype=np.int32),
-        np.asarray(tbe.row_bytes, dtype=np.int32),
+        np.asarray(tbe.row_stride, dtype=np.int32),
     )
 
 

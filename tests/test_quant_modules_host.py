@@ -219,3 +219,70 @@ def test_operator_copies_and_pickles_without_its_plans():
     back = torch.load(buf, weights_only=False)
     assert back._plans == {} and torch.equal(back.weights_dev, op.weights_dev)
     assert back.embedding_specs == op.embedding_specs and back.row_bytes == op.row_bytes
+
+
+def test_row_padding_layout_and_views():
+    """Rows of at most 128 bytes lie at the next power-of-two stride (no row straddles a
+    128-byte line) while the padded store fits the budget; every view keeps the row's width."""
+    from torchrec_amd import tbe as tbe_pkg
+    from torchrec_amd.tbe.split_table_batched_embeddings_ops_inference import (
+        IntNBitTableBatchedEmbeddingBagsCodegen as TBE,
+        line_padded_row_stride,
+    )
+
+    assert [line_padded_row_stride(w) for w in (4, 12, 16, 20, 48, 64, 68, 80, 128, 132, 144, 272)] == [
+        4, 16, 16, 32, 64, 64, 128, 128, 128, 132, 144, 272]
+    specs = [("a", 10, 128, SparseType.INT4, None), ("b", 7, 256, SparseType.INT8, None), ("c", 5, 32, SparseType.FP16, None)]
+    op = TBE(specs, device=CPU, pooling_mode=PoolingMode.SUM)  # the default: "line"
+    assert tbe_pkg.get_default_row_padding() == "line" and op.row_padding == "line"
+    assert op.row_bytes == [80, 272, 64] and op.row_stride == [128, 272, 64]
+    assert op.weights_physical_offsets == [0, 1280, 1280 + 2048] and op.weights_size == 1280 + 2048 + 512
+    op.initialize_weights()
+    for mode, widths in ((0, [80, 272, 64]), (1, [64, 256, 64]), (2, [64, 256, 64])):
+        for t, (w, s, b) in enumerate(op.split_embedding_weights_with_scale_bias(mode)):
+            assert w.shape == (specs[t][1], widths[t]) and w.stride() == (op.row_stride[t], 1)
+            assert w.untyped_storage().data_ptr() == op.weights_dev.untyped_storage().data_ptr()
+    w, scale, bias = op.split_embedding_weights_with_scale_bias(2)[0]
+    assert scale.dtype == torch.float16 and scale.shape == (10, 1) and scale.stride(0) == 64
+    # writing through the views lands in the rows of the packed buffer, 128 bytes apart
+    w.fill_(0x21)
+    scale.fill_(1.0)
+    bias.fill_(-2.0)
+    raw = op.weights_dev[:1280].view(10, 128)
+    assert (raw[:, 4:68] == 0x21).all() and (raw[:, 80:] == 0).all() and (raw[:, 68:80] == 0).all()
+    assert raw[:, :4].reshape(-1).tolist() == [0x00, 0x3C, 0x00, 0xC0] * 10
+    # the same operator with its rows at their width
+    tight = TBE(specs, device=CPU, pooling_mode=PoolingMode.SUM, row_padding="none")
+    assert tight.row_stride == tight.row_bytes == [80, 272, 64] and tight.weights_size == 1024 + 2048 + 512
+    # assigning weights gives the same table contents in either layout
+    tight.initialize_weights()
+    tight.assign_embedding_weights([(a, b) for a, b in op.split_embedding_weights(True)])
+    for (x, xs), (y, ys) in zip(op.split_embedding_weights(True), tight.split_embedding_weights(True)):
+        assert torch.equal(x, y) and (xs is None or torch.equal(xs, ys))
+    with pytest.raises(ValueError, match="row_padding"):
+        TBE(specs, device=CPU, row_padding="page")
+
+
+def test_row_padding_budget_and_default_switch(monkeypatch):
+    """An operator whose padded store would exceed the budget keeps its rows at their width
+    (the 68-byte rows of a 136 GB store stay 68 bytes apart); the default can be switched."""
+    from torchrec_amd import tbe as tbe_pkg
+    from torchrec_amd.tbe import split_table_batched_embeddings_ops_inference as mod
+
+    big = [("t", 250_000_000, 128, SparseType.INT4, None)] * 8
+    op = mod.IntNBitTableBatchedEmbeddingBagsCodegen(
+        [(f"t{i}",) + s[1:] for i, s in enumerate(big)], device=torch.device("meta"), row_alignment=4)
+    assert op.row_bytes == [68] * 8 and op.row_stride == [68] * 8 and op.weights_size == 136_000_000_000
+    monkeypatch.setattr(mod, "ROW_PADDING_BUDGET_BYTES", 1000)
+    small = mod.IntNBitTableBatchedEmbeddingBagsCodegen([("t", 10, 128, SparseType.INT4, None)], device=CPU)
+    assert small.row_stride == [80]  # 10 x 128 bytes would not fit a budget of 1000
+    monkeypatch.undo()
+    previous = tbe_pkg.set_default_row_padding("none")
+    try:
+        assert previous == "line"
+        assert mod.IntNBitTableBatchedEmbeddingBagsCodegen([("t", 10, 128, SparseType.INT4, None)], device=CPU).row_stride == [80]
+    finally:
+        tbe_pkg.set_default_row_padding(previous)
+    assert mod.IntNBitTableBatchedEmbeddingBagsCodegen([("t", 10, 128, SparseType.INT4, None)], device=CPU).row_stride == [128]
+    with pytest.raises(ValueError):
+        tbe_pkg.set_default_row_padding("page")

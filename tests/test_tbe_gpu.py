@@ -23,8 +23,13 @@ ST = {O.FP32: SparseType.FP32, O.FP16: SparseType.FP16, O.INT8: SparseType.INT8,
 POOL = {O.SUM: PoolingMode.SUM, O.MEAN: PoolingMode.MEAN, O.NONE: PoolingMode.NONE}
 
 
-def build(rng, specs, ftm, pooling, out_dtype, row_alignment):
-    """specs: [(dtype, rows, dim)].  Returns (TBE on GPU, oracle Store)."""
+def build(rng, specs, ftm, pooling, out_dtype, row_alignment, row_padding=None):
+    """specs: [(dtype, rows, dim)].  Returns (TBE on GPU, oracle Store).  The packed store's row
+    padding (rows of up to 128 bytes at a power-of-two stride, or every row at its width) is drawn
+    from the test's generator unless given: the oracle has its own copy of the tables, so the
+    lookups must not depend on it."""
+    if row_padding is None:
+        row_padding = ("line", "none")[int(rng.integers(2))]
     datas = [make_table(rng, dt, rows, dim) for dt, rows, dim in specs]
     store = O.pack_store([(dt, dim, d) for (dt, _, dim), d in zip(specs, datas)], row_alignment=row_alignment)
     weight_lists = []
@@ -35,7 +40,7 @@ def build(rng, specs, ftm, pooling, out_dtype, row_alignment):
     tbe = TBE(
         embedding_specs=[(f"t{i}", rows, dim, ST[dt], EmbeddingLocation.DEVICE) for i, (dt, rows, dim) in enumerate(specs)],
         feature_table_map=ftm, pooling_mode=POOL[pooling], device=DEV, weight_lists=weight_lists,
-        output_dtype=ST[out_dtype], row_alignment=row_alignment,
+        output_dtype=ST[out_dtype], row_alignment=row_alignment, row_padding=row_padding,
     )
     return tbe, store
 
@@ -1006,6 +1011,7 @@ def test_table_beyond_2_31_rows(tuning):
     tbe = TBE(embedding_specs=[("big", rows, 1, SparseType.FP32, EmbeddingLocation.DEVICE)],
               pooling_mode=PoolingMode.SUM, device=DEV, output_dtype=SparseType.FP32, row_alignment=4)
     tbe.initialize_weights()
+    assert tbe.row_stride == [4]
     w = tbe.weights_dev.view(torch.float32)
     assert w.numel() >= rows
     w.zero_()

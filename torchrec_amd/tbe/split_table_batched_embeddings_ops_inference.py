@@ -10,7 +10,15 @@ Storage and lookup are this package's own:
 * one ``uint8`` buffer per group holds every table; table ``t`` starts at a
   256-byte aligned offset; a row is ``[fp16 scale][fp16 bias][payload][pad]``
   for INT8/INT4/INT2 and ``[payload][pad]`` for FP16/FP32, padded to
-  ``row_alignment`` bytes;
+  ``row_alignment`` bytes (its *width*, what every view of the table shows);
+* rows lie ``row_stride`` bytes apart.  HBM is fetched in 128-byte lines, so a
+  random row costs the lines it touches: an 80-byte row at an 80-byte stride
+  straddles two lines half of the time.  With row padding "line" (the default)
+  a row of at most 128 bytes is stored at the next power-of-two stride, where
+  it never straddles a line, as long as the padded store of the operator stays
+  within ``ROW_PADDING_BUDGET_BYTES``; otherwise, and with row padding "none",
+  the stride is the width.  Views of a table are ``[rows, width]`` slices of
+  the strided buffer either way;
 * ``forward`` launches the HIP gather/dequantize/pool kernels of
   ``libtorchrec_amd.so`` on the current stream.  There is no host lookup: on a
   CPU device the module can be built, inspected and (de)serialized, but
@@ -37,6 +45,39 @@ _FORWARD_LENGTHS = None  # the library's tra_tbe_forward_lengths, bound on first
 
 _SUPPORTED_WEIGHTS = (SparseType.FP32, SparseType.FP16, SparseType.INT8, SparseType.INT4, SparseType.INT2)
 _TABLE_ALIGNMENT = 256
+_LINE_BYTES = 128
+# Row padding trades spare HBM for bandwidth; an operator whose padded store would exceed this
+# keeps its rows at their width (a fixed figure, not a share of the device's memory: the layout
+# of an operator must not depend on where it was built).
+ROW_PADDING_BUDGET_BYTES = 64 << 30
+_ROW_PADDING_MODES = ("line", "none")
+_default_row_padding = os.environ.get("TORCHREC_AMD_ROW_PADDING", "line")
+if _default_row_padding not in _ROW_PADDING_MODES:
+    raise ValueError(f"TORCHREC_AMD_ROW_PADDING={_default_row_padding!r}: expected one of {_ROW_PADDING_MODES}")
+
+
+def set_default_row_padding(mode: str) -> str:
+    """Row padding of operators built from now on ("line" or "none"); returns the previous default."""
+    global _default_row_padding
+    if mode not in _ROW_PADDING_MODES:
+        raise ValueError(f"row padding {mode!r}: expected one of {_ROW_PADDING_MODES}")
+    previous, _default_row_padding = _default_row_padding, mode
+    return previous
+
+
+def get_default_row_padding() -> str:
+    return _default_row_padding
+
+
+def line_padded_row_stride(row_bytes: int) -> int:
+    """Distance between rows of ``row_bytes`` bytes under row padding "line": the next power
+    of two for rows of at most one 128-byte line, the width for wider rows."""
+    if row_bytes > _LINE_BYTES:
+        return row_bytes
+    stride = 4
+    while stride < row_bytes:
+        stride *= 2
+    return stride
 
 
 def round_up(a: int, b: int) -> int:
@@ -72,6 +113,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         row_alignment: Optional[int] = None,
         uvm_host_mapped: bool = False,
         feature_names_per_table: Optional[List[List[str]]] = None,
+        row_padding: Optional[str] = None,
         **unsupported,
     ) -> None:
         super().__init__()
@@ -132,19 +174,34 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self.D_offsets: List[int] = D_offsets
         self.total_D: int = D_offsets[-1]
 
+        # row_bytes: width of a row (header, payload, padding to row_alignment); row_stride: distance
+        # between rows in the packed buffer (>= width, see the module docstring).
         self.row_bytes: List[int] = []
-        self.weights_physical_offsets: List[int] = []
-        total = 0
-        for r, d, ty in zip(rows, dims, self.weight_tys):
+        for d, ty in zip(dims, self.weight_tys):
             rb = rounded_row_size_in_bytes(d, ty, self.row_alignment, self.scale_bias_size_in_bytes)
             if device.type == "cuda" and rb % 4 != 0:
                 raise ValueError(
                     f"row_alignment {self.row_alignment} gives {rb}-byte rows; the GPU kernels need a multiple of 4"
                 )
             self.row_bytes.append(rb)
-            self.weights_physical_offsets.append(total)
-            total = round_up(total + r * rb, _TABLE_ALIGNMENT)
-        self.weights_size: int = total
+        self.row_padding: str = _default_row_padding if row_padding is None else row_padding
+        if self.row_padding not in _ROW_PADDING_MODES:
+            raise ValueError(f"row_padding {self.row_padding!r}: expected one of {_ROW_PADDING_MODES}")
+
+        def layout(strides: List[int]) -> Tuple[List[int], int]:
+            offsets, total = [], 0
+            for r, st in zip(rows, strides):
+                offsets.append(total)
+                total = round_up(total + r * st, _TABLE_ALIGNMENT)
+            return offsets, total
+
+        self.row_stride: List[int] = list(self.row_bytes)
+        self.weights_physical_offsets, self.weights_size = layout(self.row_stride)
+        if self.row_padding == "line":
+            padded = [line_padded_row_stride(rb) for rb in self.row_bytes]
+            offsets, total = layout(padded)
+            if total <= ROW_PADDING_BUDGET_BYTES:
+                self.row_stride, self.weights_physical_offsets, self.weights_size = padded, offsets, total
         self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
         self._identity_positions: Tuple[int, ...] = tuple(range(len(self.feature_table_map)))
         self._num_keys: Dict[Tuple[int, ...], int] = {}
@@ -188,8 +245,10 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         return n
 
     def _rows_view(self, t: int) -> Tensor:
-        off, r, rb = self.weights_physical_offsets[t], self.rows[t], self.row_bytes[t]
-        return self.weights_dev.detach()[off : off + r * rb].view(r, rb)
+        """Table ``t`` as ``[rows, row_bytes]`` bytes of the packed buffer (rows ``row_stride`` apart)."""
+        off, r, rb, st = self.weights_physical_offsets[t], self.rows[t], self.row_bytes[t], self.row_stride[t]
+        view = self.weights_dev.detach()[off : off + r * st].view(r, st)
+        return view if st == rb else view[:, :rb]
 
     def split_embedding_weights_with_scale_bias(
         self, split_scale_bias_mode: int = 1
@@ -284,7 +343,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 specs[t].rows = self.rows[t]
                 specs[t].dim = self.dims[t]
                 specs[t].dtype = self.weight_tys[t].as_int()
-                specs[t].row_bytes = self.row_bytes[t]
+                specs[t].row_bytes = self.row_stride[t]
             F = len(self.feature_table_map)
             ftm = (ctypes.c_int32 * max(F, 1))(*self.feature_table_map)
             pos = None
@@ -511,5 +570,6 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
     def extra_repr(self) -> str:
         return (
             f"tables={len(self.embedding_specs)}, features={len(self.feature_table_map)}, "
-            f"pooling={self.pooling_mode.name}, bytes={self.weights_size}, row_alignment={self.row_alignment}"
+            f"pooling={self.pooling_mode.name}, bytes={self.weights_size}, row_alignment={self.row_alignment}, "
+            f"row_padding={self.row_padding}"
         )
