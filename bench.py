@@ -43,8 +43,7 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=200)
     p.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     p.add_argument("--batches", type=int, default=None,
-                   help="distinct id batches rotated through (default 32 for c2, whose 8-batch cycle half fits the "
-                        "256 MB memory-side cache and then reads 8 %% fast; 8 elsewhere: those cycles are far larger)")
+                   help="distinct id batches rotated through (default 32 for c2, 12 for c4, 8 elsewhere)")
     p.add_argument("--mode", default="eager", choices=["graph", "eager"])
     p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
     p.add_argument("--row-padding", default=None, choices=["line", "none"],
@@ -68,6 +67,9 @@ def parse_args():
                    help="c2: rank -> id through one seeded permutation per table shared by all batches (the named "
                         "workload), or through a new permutation for every batch (cold head: no row is hot in two "
                         "batches; a lower bound, not the named workload)")
+    p.add_argument("--traffic-json", action="store_true",
+                   help="with --rocprof-summary DIR: also write profiles/<config>_lookup_traffic.json from the "
+                        "FETCH_SIZE / WRITE_SIZE runs under DIR, stamped with the hash of the kernel sources")
     p.add_argument("--batch-size", type=int, default=None, help="override the workload's batch size (tuning only; result is then not the named workload)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink table rows (debug only; result is then invalid)")
     return p.parse_args()
@@ -377,6 +379,74 @@ def cpu_baseline(wl, out_gpu, seconds):
 # --------------------------------------------------------------------------
 # rocprofv3 output -> short text (the summaries kept under profiles/)
 # --------------------------------------------------------------------------
+def kernel_source_hash():
+    """Hash of the sources the kernel library is built from (``torchrec_amd/csrc`` and
+    ``include``): a stored hardware-counter profile names the hash it was measured at, and a
+    bench run says whether the tree still has it."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    files = sorted(
+        f for pat in ("torchrec_amd/csrc/*.hip", "torchrec_amd/csrc/*.h", "torchrec_amd/csrc/Makefile", "include/*.h")
+        for f in glob.glob(os.path.join(ROOT, pat))
+    )
+    for f in files:
+        h.update(os.path.relpath(f, ROOT).encode())
+        h.update(b"\0")
+        h.update(open(f, "rb").read())
+        h.update(b"\0")
+    return h.hexdigest()[:16]
+
+
+def write_traffic_json(root, config):
+    """``profiles/<config>_lookup_traffic.json`` from the FETCH_SIZE / WRITE_SIZE counter runs under
+    ``root`` (as ``--rocprof-summary`` reads them): HBM bytes per lookup call = the counters of the
+    lookup kernel instances of the timed step (those dispatched most often; a call launches each
+    once), scaled by what the same counters read for the library's 256 MiB copy kernel."""
+    import collections
+    import csv
+    import glob
+
+    per = collections.defaultdict(lambda: collections.defaultdict(list))
+    for f in sorted(glob.glob(os.path.join(root, "**", "*counter_collection.csv"), recursive=True)):
+        for r in csv.DictReader(open(f)):
+            if r["Counter_Name"] in ("FETCH_SIZE", "WRITE_SIZE"):
+                per[r["Counter_Name"]][r["Kernel_Name"].split("(")[0].replace("void ", "")].append(float(r["Counter_Value"]))
+    out = {}
+    for ctr, copied_kib in (("FETCH_SIZE", CAL_COPY_BYTES / 1024), ("WRITE_SIZE", CAL_COPY_BYTES / 1024)):
+        ks = per.get(ctr)
+        if not ks:
+            raise SystemExit(f"no {ctr} counters under {root}")
+        copy = [v for k, v in ks.items() if "tra_copy_kernel" in k]
+        if not copy:
+            raise SystemExit(f"the {ctr} run has no dispatch of the calibration copy kernel")
+        factor = copied_kib / (sum(copy[0]) / len(copy[0]))
+        lookups = {k: v for k, v in ks.items() if "tbe_pooled" in k or "tbe_nobag" in k}
+        most = max(len(v) for v in lookups.values())
+        step = {k: sum(v) / len(v) for k, v in lookups.items() if len(v) == most}
+        out[ctr] = (sum(step.values()) * 1024 * factor, factor, sorted(step))
+    fetch, ff, kernels = out["FETCH_SIZE"]
+    write, wf, _ = out["WRITE_SIZE"]
+    doc = {
+        "kernel": kernels if len(kernels) > 1 else kernels[0],
+        "workload": config,
+        "hbm_bytes_per_launch": int(round(fetch + write)),
+        "fetch_bytes": int(round(fetch)),
+        "write_bytes": int(round(write)),
+        "fetch_factor": round(ff, 4),
+        "write_factor": round(wf, 4),
+        "kernel_source_hash": kernel_source_hash(),
+        "note": "per lookup call (all its launches); counter x factor, the factor from the same counter over the "
+                "256 MiB copy kernel; kernel_source_hash covers torchrec_amd/csrc and include",
+    }
+    path = os.path.join(ROOT, "profiles", f"{config}_lookup_traffic.json")
+    with open(path, "w") as f:
+        json.dump(doc, f, indent=1)
+        f.write("\n")
+    print(f"wrote {os.path.relpath(path, ROOT)}: {doc['hbm_bytes_per_launch'] / 1e6:.1f} MB per call")
+
+
 def rocprof_summary(root):
     import collections
     import csv
@@ -502,11 +572,15 @@ def main():
     args = parse_args()
     if args.rocprof_summary:
         rocprof_summary(args.rocprof_summary)
+        if args.traffic_json:
+            write_traffic_json(args.rocprof_summary, args.config)
         return
     if args.row_alignment is None:
         args.row_alignment = 4 if args.config == "c5" else 16
     if args.batches is None:
-        args.batches = 32 if args.config == "c2" else 8
+        # (c4: more distinct id counts than the plan keeps launch geometries, so that a geometry
+        # that is looked up per exact id count would show as a miss on every call)
+        args.batches = {"c2": 32, "c4": 12}.get(args.config, 8)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
         sys.exit(2)
@@ -717,9 +791,13 @@ def main():
         try:
             stored = json.load(open(tpath))
             traffic = stored.get("hbm_bytes_per_launch")
+            now = kernel_source_hash()
             traffic_source = {
                 "file": os.path.relpath(tpath, ROOT),
-                "measured_at_commit": stored.get("measured_at_commit"),
+                "kernel_source_hash_of_profile": stored.get("kernel_source_hash"),
+                "kernel_source_hash_now": now,
+                # stale: the kernel sources (torchrec_amd/csrc, include) changed since the counters were read
+                "stale": stored.get("kernel_source_hash") != now,
                 "note": "from the stored rocprofv3 counter runs (FETCH_SIZE, WRITE_SIZE x copy-kernel calibration), not measured in this run",
             }
         except Exception:

@@ -557,3 +557,87 @@ def test_deepcopy_of_a_used_collection():
     # the copy's state_dict tensors view the copy's buffer, as the original's view the original's
     sd = twin.state_dict()
     assert all(not v.view(torch.uint8).any() for k, v in sd.items() if k.endswith(".weight"))
+
+
+def test_qebc_shared_feature_and_registered_operators_take_the_general_route():
+    """A feature that feeds two tables makes the module's feature names repeat ([a, a, b]): a KJT
+    whose keys happen to equal that list must not take the short route (it would read the second
+    table's bags from the second key).  Registered operators are called as modules and give the
+    same bits as unregistered ones."""
+    torch.manual_seed(5)
+    B = 40
+    tables = [EmbeddingBagConfig(name="t0", embedding_dim=32, num_embeddings=100, feature_names=["a"], data_type=DataType.INT4),
+              EmbeddingBagConfig(name="t1", embedding_dim=64, num_embeddings=200, feature_names=["a", "b"], data_type=DataType.INT8)]
+    m = QuantEBC(tables, False, DEV, output_dtype=torch.half)
+    assert m._feature_names == ["a", "a", "b"] and len(m._emb_modules) == 1
+    tbe = m._emb_modules[0]
+    tbe.weights_dev.copy_(torch.randint(0, 256, tbe.weights_dev.shape, dtype=torch.uint8, device=DEV))
+    for t in range(2):
+        tbe._rows_view(t)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+    la = torch.randint(0, 6, (B,), dtype=torch.int64, device=DEV)
+    lb = torch.randint(0, 6, (B,), dtype=torch.int64, device=DEV)
+    va = torch.randint(0, 100, (int(la.sum()),), dtype=torch.int64, device=DEV)
+    vb = torch.randint(0, 200, (int(lb.sum()),), dtype=torch.int64, device=DEV)
+    kjt = KeyedJaggedTensor(keys=["a", "b"], values=torch.cat([va, vb]), lengths=torch.cat([la, lb]))
+    want = m(kjt).values()
+    # the same bags written out once per use of the feature: keys == the module's feature names
+    dup = KeyedJaggedTensor(keys=["a", "a", "b"], values=torch.cat([va, va, vb]), lengths=torch.cat([la, la, lb]))
+    got = m(dup).values()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # oracle on the module's packed bytes
+    off = np.zeros(3 * B + 1, dtype=np.int64)
+    off[1:] = np.cumsum(torch.cat([la, la, lb]).cpu().numpy())
+    ref = O.tbe_forward(oracle_store_of(tbe), [0, 1, 1], B, torch.cat([va, va, vb]).cpu().numpy(), off, None, O.SUM, O.FP16)
+    assert bits_equal(want.cpu().numpy(), ref) == 0
+    # a stride that disagrees with the lengths is not silently accepted by the short route
+    single = QuantEBC(tables[1:], False, DEV, output_dtype=torch.half)
+    single._emb_modules[0].weights_dev.copy_(torch.randint(0, 256, single._emb_modules[0].weights_dev.shape, dtype=torch.uint8, device=DEV))
+    single._emb_modules[0]._rows_view(0)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+    ok = KeyedJaggedTensor(keys=["a", "b"], values=torch.cat([va, vb]) % 200, lengths=torch.cat([la, lb]))
+    base = single(ok).values()
+    with_stride = KeyedJaggedTensor(keys=["a", "b"], values=torch.cat([va, vb]) % 200, lengths=torch.cat([la, lb]), stride=B)
+    assert torch.equal(single(with_stride).values().view(torch.int16), base.view(torch.int16))
+    # registered operators: hooks fire, same bits
+    reg = QuantEBC(tables, False, DEV, output_dtype=torch.half, register_tbes=True)
+    reg._emb_modules[0].weights_dev.copy_(tbe.weights_dev)
+    fired = []
+    reg.tbes[0].register_forward_hook(lambda mod, args, out: fired.append(out.shape))
+    got = reg(kjt).values()
+    assert fired == [(B, 32 + 64 + 64)] and torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_qec_prepared_flags_and_registered_operators_give_the_same_rows():
+    """``__use_unflattened_lengths_for_batching``, ``__use_batching_hinted_output`` off,
+    ``__remove_stbe_padding`` and ``register_tbes`` change how the lookup is wrapped, not its rows."""
+    from torchrec_amd.quant import embedding_modules as qm
+
+    rng = np.random.default_rng(21)
+    t = [EmbeddingConfig(name="t1", embedding_dim=32, num_embeddings=50, feature_names=["f1", "f2"], data_type=DataType.INT8),
+         EmbeddingConfig(name="t2", embedding_dim=32, num_embeddings=70, feature_names=["f3"], data_type=DataType.INT4)]
+    base = QuantEC(t, DEV, output_dtype=torch.half, need_indices=True)
+    for op in base._emb_modules:
+        op.weights_dev.copy_(torch.randint(0, 256, op.weights_dev.shape, dtype=torch.uint8, device=DEV))
+        for i in range(len(op.rows)):
+            op._rows_view(i)[:, 0:4] = torch.tensor([0x00, 0x2C, 0x00, 0xAC], dtype=torch.uint8, device=DEV)
+    kjt = random_kjt(rng, ["f3", "f1", "f2"], [70, 50, 50], B=17, max_len=6)
+    want = base(kjt)
+    variants = []
+    for attr, value in ((qm.MODULE_ATTR_USE_UNFLATTENED_LENGTHS_FOR_BATCHING, True),
+                        (qm.MODULE_ATTR_USE_BATCHING_HINTED_OUTPUT, False),
+                        (qm.MODULE_ATTR_REMOVE_STBE_PADDING_BOOL, True)):
+        m = QuantEC(t, DEV, output_dtype=torch.half, need_indices=True)
+        setattr(m, attr, value)
+        variants.append(m)
+    variants.append(QuantEC(t, DEV, output_dtype=torch.half, need_indices=True, register_tbes=True))
+    fired = []
+    for op in variants[-1].tbes:
+        op.register_forward_pre_hook(lambda mod, args: fired.append(1))
+    for m in variants:
+        for src, dst in zip(base._emb_modules, m._emb_modules):
+            dst.weights_dev.copy_(src.weights_dev)
+        got = m(random_kjt(np.random.default_rng(21), ["f3", "f1", "f2"], [70, 50, 50], B=17, max_len=6))
+        assert got.keys() == want.keys() if hasattr(got, "keys") else True
+        for k in ("f1", "f2", "f3"):
+            assert torch.equal(got[k].values().view(torch.int16), want[k].values().view(torch.int16))
+            assert torch.equal(got[k].lengths(), want[k].lengths()) and torch.equal(got[k].weights(), want[k].weights())
+    assert len(fired) == 2

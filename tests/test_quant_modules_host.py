@@ -286,3 +286,98 @@ def test_row_padding_budget_and_default_switch(monkeypatch):
     assert mod.IntNBitTableBatchedEmbeddingBagsCodegen([("t", 10, 128, SparseType.INT4, None)], device=CPU).row_stride == [128]
     with pytest.raises(ValueError):
         tbe_pkg.set_default_row_padding("page")
+
+
+def _stub_lookups(module, calls):
+    """Stand-ins for the operators' GPU lookup: zeros into the caller's buffer, and a record of
+    whether the operator was reached through ``__call__`` (hooks fire) or through ``forward``."""
+    for i, op in enumerate(module._emb_modules):
+        def fake_forward(*args, _i=i, **kw):
+            calls.append(("forward", _i))
+            kw["out"].zero_()
+            return kw["out"]
+        op.forward = fake_forward  # type: ignore[method-assign]
+        op.register_forward_pre_hook(lambda m, a, kw=None, _i=i: calls.append(("hook", _i)))
+
+
+def test_ec_batching_hint_follows_the_prepared_lengths_form(monkeypatch):
+    """The order of the reference's graph (torchrec/quant/embedding_modules.py:943-950, pinned by
+    torchrec/quant/tests/test_embedding_modules.py:1027-1117): by default the batching hint sees
+    the flattened lengths and the lengths are unflattened afterwards; prepared with
+    ``__use_unflattened_lengths_for_batching`` the hint is a user of the unflattened lengths;
+    with ``__use_batching_hinted_output`` off (and flattened lengths) there is no hint."""
+    from torchrec_amd.quant import embedding_modules as qm
+
+    t = [EmbeddingConfig(name="t1", embedding_dim=16, num_embeddings=10, feature_names=["f1", "f2"], data_type=DataType.FP16),
+         EmbeddingConfig(name="t2", embedding_dim=16, num_embeddings=10, feature_names=["f3", "f4"], data_type=DataType.FP16)]
+    q = QuantEC(t, CPU, output_dtype=torch.half)
+    calls = []
+    _stub_lookups(q, calls)
+    seen = []
+    real_unflatten, real_hint = qm._get_unflattened_lengths, qm._get_batching_hinted_output
+    monkeypatch.setattr(qm, "_get_unflattened_lengths",
+                        lambda lengths, n: (seen.append(("unflatten", tuple(lengths.shape))), real_unflatten(lengths, n))[1])
+    monkeypatch.setattr(qm, "_get_batching_hinted_output",
+                        lambda lengths, output: (seen.append(("hint", tuple(lengths.shape))), real_hint(lengths=lengths, output=output))[1])
+    kjt = KeyedJaggedTensor(keys=["f1", "f2", "f3", "f4"], values=torch.arange(6) % 10,
+                            lengths=torch.tensor([1, 0, 2, 0, 1, 1, 0, 1]))
+    out = q(kjt)
+    assert seen == [("hint", (8,)), ("unflatten", (8,))]
+    assert [tuple(out[k].values().shape) for k in ("f1", "f2", "f3", "f4")] == [(1, 16), (2, 16), (2, 16), (1, 16)]
+    assert out["f3"].lengths().tolist() == [1, 1]
+    seen.clear()
+    setattr(q, qm.MODULE_ATTR_USE_UNFLATTENED_LENGTHS_FOR_BATCHING, True)
+    q(kjt)
+    assert seen == [("unflatten", (8,)), ("hint", (4, 2))]
+    seen.clear()
+    setattr(q, qm.MODULE_ATTR_USE_UNFLATTENED_LENGTHS_FOR_BATCHING, False)
+    setattr(q, qm.MODULE_ATTR_USE_BATCHING_HINTED_OUTPUT, False)
+    q(kjt)
+    assert seen == [("unflatten", (8,))]
+    # every lookup above went through the operators' forward (they are not registered)
+    assert calls and all(kind == "forward" for kind, _ in calls)
+
+
+def test_ec_remove_padding_drops_rows_behind_the_last_bag():
+    """``__remove_stbe_padding``: a values tensor longer than the lengths add up to (padding at
+    its end) yields per-feature rows of the bags only, and the buffer is cut at the last bag's end
+    (construct_jagged_tensors_inference(remove_padding=True), torchrec/modules/utils.py:315-316)."""
+    from torchrec_amd.quant import embedding_modules as qm
+
+    t = [EmbeddingConfig(name="t1", embedding_dim=8, num_embeddings=10, feature_names=["f1", "f2"], data_type=DataType.INT8)]
+    q = QuantEC(t, CPU, output_dtype=torch.float, need_indices=True)
+    _stub_lookups(q, [])
+    values = torch.tensor([3, 4, 5, 6, 7, 9, 9, 9])  # three entries of padding
+    kjt = KeyedJaggedTensor(keys=["f1", "f2"], values=values, lengths=torch.tensor([2, 1, 0, 2]))
+    for flag in (False, True):
+        setattr(q, qm.MODULE_ATTR_REMOVE_STBE_PADDING_BOOL, flag)
+        out = q(kjt)
+        assert out["f1"].values().shape == (3, 8) and out["f2"].values().shape == (2, 8)
+        assert out["f1"].weights().tolist() == [3, 4, 5] and out["f2"].weights().tolist() == [6, 7]
+        base = out["f1"].values()
+        rows_in_buffer = base.untyped_storage().nbytes() // (8 * 4)
+        assert rows_in_buffer == 8  # one buffer for the whole KJT either way; the views stop at row 5
+
+
+@pytest.mark.parametrize("cls", ["ebc", "ec"])
+def test_registered_operators_are_called_as_modules(cls):
+    """``register_tbes``: the operators are submodules (``tbes``) and the collection calls them
+    through ``__call__``, so hooks see every lookup; unregistered operators are reached through
+    ``forward`` (torchrec/quant/embedding_modules.py:546-557, 938-942)."""
+    for register in (False, True):
+        if cls == "ebc":
+            t = [EmbeddingBagConfig(name="t1", embedding_dim=8, num_embeddings=10, feature_names=["f1"], data_type=DataType.INT8),
+                 EmbeddingBagConfig(name="t2", embedding_dim=8, num_embeddings=10, feature_names=["f2"], data_type=DataType.INT8,
+                                    pooling=PoolingType.MEAN)]
+            q = QuantEBC(t, False, CPU, output_dtype=torch.float, register_tbes=register)
+        else:
+            t = [EmbeddingConfig(name="t1", embedding_dim=8, num_embeddings=10, feature_names=["f1"], data_type=DataType.INT8),
+                 EmbeddingConfig(name="t2", embedding_dim=8, num_embeddings=10, feature_names=["f2"], data_type=DataType.INT4)]
+            q = QuantEC(t, CPU, output_dtype=torch.float, register_tbes=register)
+        assert hasattr(q, "tbes") == register
+        calls = []
+        _stub_lookups(q, calls)
+        q(KeyedJaggedTensor(keys=["f1", "f2"], values=torch.tensor([1, 2, 3]), offsets=torch.tensor([0, 1, 2, 2, 3])))
+        kinds = [kind for kind, _ in calls]
+        assert kinds.count("forward") == 2
+        assert kinds.count("hook") == (2 if register else 0)

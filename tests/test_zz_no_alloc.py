@@ -3,7 +3,10 @@ array and the scan's partial sums) is a static device array of the library, so
 the call allocates nothing.  Called through the C ABI and compared, bit for
 bit, with tra_tbe_forward_lengths on a caller-allocated workspace: two calls in
 a row, the second on a smaller input (the array keeps the first call's
-contents), on the routes that use the scratch (scan + lookup)."""
+contents), on the routes that use the scratch (scan + lookup).  The call must
+leave the device's free memory and torch's pools as they were, and it is the
+entry for callers under HIP graph capture: a captured call is replayed several
+times, with eager work in between, against the eager result."""
 import ctypes
 
 import numpy as np
@@ -50,7 +53,15 @@ def _both_entries(tbe, ids, lengths, B, K, total_D):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
     args = (plan, _lib.ptr(tbe.weights_dev), _lib.ptr(ti), _lib.ptr(tl), 0, None, B, K, len(ids),
             _lib.POOL_SUM, _lib.FP16)
+    # the static entry allocates nothing: neither from the device (hipMemGetInfo) nor from torch's pools
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(DEV)
+    reserved_before, allocated_before = torch.cuda.memory_reserved(DEV), torch.cuda.memory_allocated(DEV)
     _lib.check(lib.tra_tbe_forward_lengths_static(*args, out_static.data_ptr(), total_D, stream))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(DEV)
+    assert free_after == free_before
+    assert (torch.cuda.memory_reserved(DEV), torch.cuda.memory_allocated(DEV)) == (reserved_before, allocated_before)
     _lib.check(lib.tra_tbe_forward_lengths(*args, out_ws.data_ptr(), total_D, ws.data_ptr(), stream))
     torch.cuda.synchronize()
     return out_static.cpu().numpy(), out_ws.cpu().numpy()
@@ -92,3 +103,60 @@ def test_static_scratch_entry_refuses_what_does_not_fit():
                                             _lib.current_stream(DEV))
     assert rc == -5  # TRA_ERR_TOO_LARGE, nothing launched
     assert b"static" in lib.tra_last_error()
+
+
+def test_static_scratch_entry_under_graph_capture():
+    """The context the entry is for: captured in a HIP graph (a scan + lookup call, more than
+    16384 bags, so the scratch is used), replayed four times with new inputs and eager work
+    between the replays; every replay equals the workspace entry run eagerly on the same inputs."""
+    rng = np.random.default_rng(99)
+    specs = [(O.INT4, 3000, 64), (O.INT8, 2500, 64), (O.INT4, 2000, 64), (O.INT8, 1500, 64)]
+    tbe, _ = _operator(rng, specs)
+    K, total_D, B = len(specs), 64 * len(specs), 6000
+    assert K * B > 16384
+    rows_f = [s[1] for s in specs]
+    lib = _lib.lib()
+    plan = tbe._get_plan(None)
+    cap = K * B * 5
+    ti = torch.zeros(cap, dtype=torch.int32, device=DEV)
+    tl = torch.zeros(K * B, dtype=torch.int32, device=DEV)
+    out = torch.zeros(B, total_D, dtype=torch.float16, device=DEV)
+    ws = torch.empty(lib.tra_tbe_forward_lengths_workspace_bytes(K, B, 0), dtype=torch.uint8, device=DEV)
+
+    def load(seed):
+        lengths, _, ids = make_bags(np.random.default_rng(seed), rows_f, B, 5)
+        ti.zero_()
+        ti[: len(ids)].copy_(torch.from_numpy(ids))
+        tl.copy_(torch.from_numpy(lengths))
+        return len(ids)
+
+    # the captured call reads its id count from the launch arguments: every replay uses inputs
+    # padded to the same count (ids past the bags are never read)
+    n0 = load(0)
+    n_ids = cap
+
+    def call_static(stream):
+        _lib.check(lib.tra_tbe_forward_lengths_static(plan, _lib.ptr(tbe.weights_dev), _lib.ptr(ti), _lib.ptr(tl), 0, None,
+                                                      B, K, n_ids, _lib.POOL_SUM, _lib.FP16, out.data_ptr(), total_D, stream))
+
+    call_static(_lib.current_stream(DEV))  # geometry of this call shape, outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            call_static(_lib.current_stream(DEV))
+    torch.cuda.synchronize()
+    assert n0 <= cap
+    for seed in (1, 2, 3, 4):
+        load(seed)
+        out.fill_(3.0)
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().copy()
+        eager = torch.full((B, total_D), 5.0, dtype=torch.float16, device=DEV)
+        _lib.check(lib.tra_tbe_forward_lengths(plan, _lib.ptr(tbe.weights_dev), _lib.ptr(ti), _lib.ptr(tl), 0, None, B, K,
+                                               n_ids, _lib.POOL_SUM, _lib.FP16, eager.data_ptr(), total_D, ws.data_ptr(),
+                                               _lib.current_stream(DEV)))
+        torch.cuda.synchronize()
+        assert bits_equal(got, eager.cpu().numpy()) == 0, seed

@@ -371,12 +371,14 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
       // Blocks are dealt to the dies round-robin; the remap assumes every die
       // has the same number of CUs.  Anything else: no remap.
       plan->num_xcd = (xcds >= 1 && cus % xcds == 0) ? xcds : 1;
-      const int rc = resolve_static_scratch(plan->device);
-      if (rc != TRA_OK) {
-        delete plan;
-        return rc;
+      // Only tra_tbe_forward_lengths_static needs the static scratch: where it cannot be
+      // resolved the plan is still good for every other entry point, and that one reports it.
+      if (resolve_static_scratch(plan->device) == TRA_OK) {
+        plan->static_scratch = g_scratch_ptr[plan->device];
+      } else {
+        (void)hipGetLastError();
+        plan->static_scratch = nullptr;
       }
-      plan->static_scratch = g_scratch_ptr[plan->device];
     }
   }
   size_t total = 0;
@@ -626,6 +628,18 @@ static void compute_geometry(const tra_tbe* tbe, const Tuning& tune, bool balanc
   }
 }
 
+// The grid of a sequence lookup follows the number of ids, which differs from call to call in
+// service.  Geometries are kept per id count rounded up to a step of an eighth of its power of
+// two (the blocks of a feature stride over its ids, so any grid of about the right size will
+// do): neighbouring batch sizes share an entry instead of each evicting one.
+static int64_t quantized_id_count(int64_t n) {
+  if (n <= 1024) return 1024;
+  int lg = 0;
+  while ((int64_t(1) << (lg + 1)) <= n) ++lg;
+  const int64_t step = int64_t(1) << (lg - 3);
+  return (n + step - 1) / step * step;
+}
+
 static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
                         const void* offsets, bool from_lengths, int32_t idx_is_i64,
                         const float* per_sample_weights, int32_t batch_size, int64_t num_indices,
@@ -690,15 +704,16 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     const int gen = g_ovr_gen.load(std::memory_order_relaxed);
     const Tuning tune = choose_tuning(tbe->num_cus, (int64_t)tbe->num_features * batch_size, num_indices);
     const int balanced = use_window_kernel(tbe, tune, nobag, batch_size) ? 1 : 0;
+    const int64_t geo_indices = nobag ? quantized_id_count(num_indices) : num_indices;
     for (const auto& g : tbe->geo)
       if (g && g->batch_size == batch_size && g->gen == gen && g->balanced == balanced &&
-          g->nobag == (int)nobag && (!nobag || g->nobag_indices == num_indices)) {
+          g->nobag == (int)nobag && (!nobag || g->nobag_indices == geo_indices)) {
         geo = g;
         break;
       }
     if (!geo) {
       auto g = std::make_shared<Geometry>();
-      compute_geometry(tbe, tune, balanced != 0, nobag, batch_size, num_indices, *g);
+      compute_geometry(tbe, tune, balanced != 0, nobag, batch_size, geo_indices, *g);
       g->gen = gen;
       geo = g;
       tbe->geo[tbe->geo_next] = geo;  // a call still launching from the replaced entry keeps it alive

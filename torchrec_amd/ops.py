@@ -110,7 +110,12 @@ def length_per_key_async(lengths: torch.Tensor, num_features: int, stride: int):
         arrived = torch.cuda.Event()
         arrived.record(side)
 
-    def finish() -> List[int]:
+    # The side stream reads ``lengths`` (possibly a contiguous copy made above, which nobody else
+    # holds): the allocator is told so, and the returned function keeps the tensor until the copy
+    # has arrived, so that its memory is not handed to a later allocation of the current stream.
+    lengths.record_stream(side)
+
+    def finish(_held=lengths) -> List[int]:
         arrived.synchronize()
         return host.tolist()
 

@@ -451,7 +451,13 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         # Everything the general route below would establish is checked here
         # in a few attribute reads, and the operator is launched directly.
         ops_ = self._emb_modules
-        if len(ops_) == 1 and not self._is_weighted and position_weights is None and features._offsets is None:
+        if (
+            len(ops_) == 1
+            and not self._is_weighted
+            and position_weights is None
+            and features._offsets is None
+            and not self.register_tbes  # (registered operators are called as modules, below)
+        ):
             op = ops_[0]
             v, ln, keys = features._values, features._lengths, features._keys
             if (
@@ -461,6 +467,7 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
                 and ln.is_cuda
                 and (v.dtype is torch.int64 or v.dtype is torch.int32)
                 and ln.dtype is v.dtype
+                and ln.device == v.device
                 and ln.dim() == 1
                 and v.is_contiguous()
                 and ln.is_contiguous()
@@ -471,7 +478,15 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
             ):
                 K = len(keys)
                 B = ln.numel() // K if K else 0
-                if B > 0 and ln.numel() == K * B:
+                # (a feature that feeds two tables appears twice among the module's feature names: its
+                # bags are then read twice from one key, which the general route below resolves)
+                if (
+                    B > 0
+                    and ln.numel() == K * B
+                    and features._stride in (None, B)
+                    and features._stride_per_key is None
+                    and self._feature_names_unique()
+                ):
                     out = torch.empty(B, self._total_D, dtype=self._output_dtype, device=v.device)
                     op._launch_from_lengths(
                         None, v, ln, int(v.dtype is torch.int64), None, B, K, v.numel(), out.data_ptr(), out.stride(0)
@@ -497,7 +512,10 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         out = torch.empty((B, self._total_D), dtype=self._output_dtype, device=indices.device)
         col = 0
         for emb_op, positions in zip(self._emb_modules, self._group_positions(order)):
-            emb_op.forward(  # type: ignore[operator]
+            # An operator registered as a submodule (register_tbes) is called as a module, so that
+            # hooks and leaf-module tracing see the call (torchrec/quant/embedding_modules.py:546-557).
+            call = emb_op if self.register_tbes else emb_op.forward
+            call(  # type: ignore[operator]
                 indices=indices,
                 offsets=offsets,
                 lengths=lengths,
@@ -510,6 +528,12 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
             )
             col += emb_op.total_D  # type: ignore[union-attr]
         return KeyedTensor(keys=self._embedding_names, values=out, length_per_key=self._length_per_key)
+
+    def _feature_names_unique(self) -> bool:
+        unique = getattr(self, "_feature_names_are_unique", None)
+        if unique is None:
+            unique = self._feature_names_are_unique = len(set(self._feature_names)) == len(self._feature_names)
+        return unique
 
     def _get_name(self) -> str:
         return "QuantizedEmbeddingBagCollection"
@@ -751,7 +775,7 @@ class EmbeddingCollection(EmbeddingCollectionInterface, ModuleNoCopyMixin, _Feat
         B = features.stride()
         indices = features.values()
         offsets = features.offsets()
-        lengths = features.lengths().view(len(kjt_keys), -1) if kjt_keys else features.lengths()
+        lengths = features.lengths()
         L = indices.numel()
         # Row ranges of the input keys: one small device-to-host copy.  Where the
         # KJT does not carry the per-key counts, their reduction and copy are
@@ -771,21 +795,42 @@ class EmbeddingCollection(EmbeddingCollectionInterface, ModuleNoCopyMixin, _Feat
         else:
             offset_per_key = features.offset_per_key()
         lookup = torch.empty((L, self._embedding_dim), dtype=self._output_dtype, device=indices.device)
-        f0 = 0
-        for emb_module, n_feat in zip(self._emb_modules, self._feature_splits):
-            emb_module.forward(
-                indices=indices,
-                offsets=offsets,
-                feature_positions=order[f0 : f0 + n_feat],
-                batch_size=B,
-                out=lookup,
-            )
-            f0 += n_feat
+        try:
+            f0 = 0
+            for emb_module, n_feat in zip(self._emb_modules, self._feature_splits):
+                # (a registered operator is called as a module, torchrec/quant/embedding_modules.py:938-942)
+                call = emb_module if self.register_tbes else emb_module.forward
+                call(
+                    indices=indices,
+                    offsets=offsets,
+                    feature_positions=order[f0 : f0 + n_feat],
+                    batch_size=B,
+                    out=lookup,
+                )
+                f0 += n_feat
+        finally:
+            # The reduction queued on the side stream reads the KJT's lengths: it is waited for
+            # also when a lookup raises, before anything of this call is released.
+            if counts_later is not None:
+                features._length_per_key = counts_later()  # the KJT remembers them, as length_per_key() would
         if counts_later is not None:
-            features._length_per_key = counts_later()  # the KJT remembers them, as length_per_key() would
             offset_per_key = features.offset_per_key()
-        if getattr(self, MODULE_ATTR_USE_BATCHING_HINTED_OUTPUT, True):
+        # The batching hint sees the flattened lengths by default and the [F, B] lengths when the
+        # module is prepared for it (torchrec/quant/embedding_modules.py:943-950); here the lengths
+        # are those of the whole KJT, because all operators write one buffer.
+        if getattr(self, MODULE_ATTR_USE_UNFLATTENED_LENGTHS_FOR_BATCHING, False):
+            if kjt_keys:
+                lengths = _get_unflattened_lengths(features.lengths(), len(kjt_keys))
             lookup = _get_batching_hinted_output(lengths=lengths, output=lookup)
+        else:
+            if getattr(self, MODULE_ATTR_USE_BATCHING_HINTED_OUTPUT, True):
+                lookup = _get_batching_hinted_output(lengths=features.lengths(), output=lookup)
+            if kjt_keys:
+                lengths = _get_unflattened_lengths(features.lengths(), len(kjt_keys))
+        if getattr(self, MODULE_ATTR_REMOVE_STBE_PADDING_BOOL, False):
+            # Rows past the last id that belongs to a bag (a padded values tensor) are dropped
+            # (construct_jagged_tensors_inference(remove_padding=True), torchrec/modules/utils.py:315-316).
+            lookup = lookup[: offset_per_key[-1]]
         lengths_rows = torch.unbind(lengths, dim=0) if kjt_keys else ()
         feature_embeddings: Dict[str, JaggedTensor] = {}
         f = 0
