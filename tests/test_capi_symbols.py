@@ -68,3 +68,27 @@ def test_more_argument_errors():
     assert l.tra_tbe_launch_info(None, 1, 1, 0, 0, None, 0) == -1
     n = i64(0)
     assert l.tra_tbe_error_count(None, None, ctypes.byref(n)) == -1
+
+
+def test_fastcall_module_binds_the_same_entry_point():
+    """The extension module in front of tra_tbe_forward_lengths: built with the library, takes the
+    entry point's address from Python, and refuses anything but fifteen integer arguments.  (No
+    compute call here: that needs a GPU.)"""
+    import ctypes
+
+    from torchrec_amd import _fastcall
+
+    lib = _lib.lib()
+    address = ctypes.cast(lib.tra_tbe_forward_lengths, ctypes.c_void_p).value
+    assert address
+    fn = _lib.forward_lengths_entry()
+    assert fn is _fastcall.forward_lengths
+    import pytest
+
+    with pytest.raises(TypeError):
+        fn(1, 2, 3)
+    with pytest.raises(TypeError):
+        fn(*(["x"] * 15))
+    # a null plan is refused by the entry point itself, with its usual code and message
+    rc = fn(None, None, None, None, 0, None, 1, 1, 0, _lib.POOL_SUM, _lib.FP16, None, 0, None, None)
+    assert rc < 0 and b"null plan" in lib.tra_last_error()

@@ -130,6 +130,20 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+def forward_lengths_entry():
+    """``tra_tbe_forward_lengths`` as a callable of fifteen integers (addresses as ints, ``None`` for
+    a null pointer) returning the entry point's code.  The in-tree extension module ``_fastcall``
+    (built with the library; it reads the integers straight from the argument vector) when it is
+    there, else the ctypes function: the same symbol of the same library either way."""
+    l = lib()
+    try:
+        from torchrec_amd import _fastcall
+    except ImportError:
+        return l.tra_tbe_forward_lengths
+    _fastcall.bind(ctypes.cast(l.tra_tbe_forward_lengths, ctypes.c_void_p).value)
+    return _fastcall.forward_lengths
+
+
 def check(rc: int) -> None:
     if rc != TRA_OK:
         msg = lib().tra_last_error().decode("utf-8", "replace")

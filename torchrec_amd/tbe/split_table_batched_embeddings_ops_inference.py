@@ -203,6 +203,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             if total <= ROW_PADDING_BUDGET_BYTES:
                 self.row_stride, self.weights_physical_offsets, self.weights_size = padded, offsets, total
         self._plans: Dict[Optional[Tuple[int, ...]], ctypes.c_void_p] = {}
+        self._plan_address: Dict[Optional[Tuple[int, ...]], int] = {}  # the same handles as integers
         self._identity_positions: Tuple[int, ...] = tuple(range(len(self.feature_table_map)))
         self._num_keys: Dict[Tuple[int, ...], int] = {}
         self._workspace: Dict[int, Tensor] = {}  # per stream: scratch of forward(offsets=None, lengths=...)
@@ -317,6 +318,9 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
                 except Exception:  # interpreter shutdown
                     pass
             plans.clear()
+        addresses = getattr(self, "_plan_address", None)
+        if addresses:
+            addresses.clear()
 
     def __del__(self) -> None:
         self._drop_plan()
@@ -327,6 +331,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         and are made again on the copy's first lookup."""
         state = self.__dict__.copy()
         state["_plans"] = {}
+        state["_plan_address"] = {}
         state["_workspace"] = {}
         state["_ws_ptr"] = {}
         return state
@@ -543,9 +548,13 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         global _FORWARD_LENGTHS
         fn = _FORWARD_LENGTHS
         if fn is None:
-            fn = _FORWARD_LENGTHS = _lib.lib().tra_tbe_forward_lengths
+            fn = _FORWARD_LENGTHS = _lib.forward_lengths_entry()
+        # (fn takes the plan's address as an integer: the extension module reads plain ints)
+        plan = self._plan_address.get(positions)
+        if plan is None:
+            plan = self._plan_address[positions] = self._get_plan(positions).value
         rc = fn(
-            self._get_plan(positions), self._buffers["weights_dev"].data_ptr(), indices.data_ptr(),
+            plan, self._buffers["weights_dev"].data_ptr(), indices.data_ptr(),
             lengths.data_ptr(), i64, None if psw is None else psw.data_ptr(), B, k_total, L,
             int(self.pooling_mode), self.output_dtype, out_ptr, out_stride, ws_ptr, stream,
         )
