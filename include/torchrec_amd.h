@@ -44,8 +44,10 @@ extern "C" {
  * uint8 buffer; table t starts at byte `offset`; row r starts at
  * offset + r * row_bytes.  INT8/INT4/INT2 rows are
  *   [fp16 scale][fp16 bias][payload dim*bits/8 bytes][pad]
- * FP16/FP32 rows are [payload][pad].  row_bytes and offset must be multiples
- * of 4.  (Reference: embedding_specs + row_alignment handed to
+ * FP16/FP32 rows are [payload][pad].  row_bytes is the distance between rows:
+ * at least header + payload, and as much padding behind a row as the caller
+ * likes (a 68-byte row stored every 128 bytes never straddles a 128-byte HBM
+ * line).  row_bytes and offset must be multiples of 4.  (Reference: embedding_specs + row_alignment handed to
  * IntNBitTableBatchedEmbeddingBagsCodegen, torchrec/quant/embedding_modules.py:
  * 393-435.) */
 typedef struct tra_table_spec {
