@@ -381,3 +381,42 @@ def test_registered_operators_are_called_as_modules(cls):
         kinds = [kind for kind, _ in calls]
         assert kinds.count("forward") == 2
         assert kinds.count("hook") == (2 if register else 0)
+
+
+@pytest.mark.parametrize("split", [False, True])
+def test_state_dict_moves_between_row_paddings(split):
+    """A state dict saved from a collection whose rows lie at their width loads into one whose rows
+    are line-padded (and back): the buffers have the same names and shapes in either layout, and
+    the table contents (payload, scale, bias of every row) arrive unchanged."""
+    from torchrec_amd import tbe as tbe_pkg
+
+    tables = [
+        EmbeddingBagConfig(name="t4", embedding_dim=128, num_embeddings=12, feature_names=["a"], data_type=DataType.INT4),
+        EmbeddingBagConfig(name="t8", embedding_dim=32, num_embeddings=9, feature_names=["b"], data_type=DataType.INT8),
+        EmbeddingBagConfig(name="th", embedding_dim=16, num_embeddings=7, feature_names=["c"], data_type=DataType.FP16),
+    ]
+
+    def build(padding):
+        previous = tbe_pkg.set_default_row_padding(padding)
+        try:
+            return QuantEBC(tables, False, CPU, quant_state_dict_split_scale_bias=split)
+        finally:
+            tbe_pkg.set_default_row_padding(previous)
+
+    tight, padded = build("none"), build("line")
+    assert tight._emb_modules[0].row_stride == [80, 48, 32] and padded._emb_modules[0].row_stride == [128, 64, 32]
+    gen = torch.Generator().manual_seed(3)
+    src = tight._emb_modules[0]
+    src.weights_dev.copy_(torch.randint(0, 256, src.weights_dev.shape, dtype=torch.uint8, generator=gen))
+    sd = tight.state_dict()
+    assert {k: tuple(v.shape) for k, v in sd.items()} == {k: tuple(v.shape) for k, v in padded.state_dict().items()}
+    padded.load_state_dict(sd)
+    contents = lambda m: [(w.clone(), None if s is None else s.clone())
+                          for w, s in m._emb_modules[0].split_embedding_weights(True)]
+    for (w0, s0), (w1, s1) in zip(contents(tight), contents(padded)):
+        assert torch.equal(w0, w1) and (s0 is None or torch.equal(s0, s1))
+    # and back into a fresh tight collection
+    again = build("none")
+    again.load_state_dict(padded.state_dict())
+    for (w0, s0), (w1, s1) in zip(contents(tight), contents(again)):
+        assert torch.equal(w0, w1) and (s0 is None or torch.equal(s0, s1))

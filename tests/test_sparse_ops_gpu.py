@@ -15,7 +15,7 @@ DEV = torch.device("cuda:0")
 
 
 @pytest.mark.parametrize("n", [0, 1, 2, 63, 64, 65, 2047, 2048, 2049, 4095, 4096, 4097, 53_248, 100_003,
-                               131_071, 131_072, 131_073, 1_048_577])
+                               131_071, 131_072, 131_073, 200_001, 262_143, 262_144, 262_145, 1_048_577])
 @pytest.mark.parametrize("dtype", [np.int32, np.int64])
 def test_cumsum(n, dtype):
     rng = np.random.default_rng(n)

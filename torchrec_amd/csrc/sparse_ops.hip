@@ -76,9 +76,30 @@ __global__ __launch_bounds__(kSmallThreads) void scan_small_kernel(const T* __re
   const int t = threadIdx.x;
   int64_t pre = 0;
   if (VEC) {
+    // The tiles in front of this block's: sixteen loads in flight per thread (the last block of
+    // a 64-tile input reads 63 tiles; one load at a time would be 63 round trips).
     const Vec* vin = reinterpret_cast<const Vec*>(in);
-#pragma unroll 4
-    for (int k = 0; k < (int)blockIdx.x; ++k) {
+    const int nk = (int)blockIdx.x;
+    int k = 0;
+    for (; k + 16 <= nk; k += 16) {
+      Vec x[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) x[j] = vin[(int64_t)(k + j) * kSmallThreads + t];
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+#pragma unroll
+        for (int i = 0; i < V; ++i) pre += (int64_t)x[j].v[i];
+    }
+    for (; k + 4 <= nk; k += 4) {
+      Vec x[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = vin[(int64_t)(k + j) * kSmallThreads + t];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < V; ++i) pre += (int64_t)x[j].v[i];
+    }
+    for (; k < nk; ++k) {
       const Vec x = vin[(int64_t)k * kSmallThreads + t];
 #pragma unroll
       for (int i = 0; i < V; ++i) pre += (int64_t)x.v[i];
@@ -784,8 +805,12 @@ using namespace tra;
 
 extern "C" {
 
-// Longest input the one-launch scan takes (64 tiles of int64, 32 of int32).
+// The one-launch scan takes inputs of up to 64 tiles of 1024 x 16 bytes: 131072 int64 or 262144
+// int32 lengths.  (The workspace size does not know the width and covers the narrower limit.)
 constexpr int64_t kSmallScanMax = (int64_t)kSmallMaxTiles * kSmallThreads * 2;
+static bool one_launch_scan(int64_t n, int32_t is_i64) {
+  return n <= (int64_t)kSmallMaxTiles * kSmallThreads * (is_i64 ? 2 : 4);
+}
 
 int64_t tra_cumsum_workspace_bytes(int64_t n) {
   if (n <= kSmallScanMax) return 0;
@@ -804,7 +829,7 @@ int tra_cumsum(const void* lengths, int64_t n, int32_t is_i64, void* offsets, vo
     return TRA_ERR_TOO_LARGE;
   }
   hipStream_t s = (hipStream_t)stream;
-  if (n <= kSmallScanMax) {
+  if (one_launch_scan(n, is_i64)) {
     const int per_tile = kSmallThreads * (is_i64 ? 2 : 4);
     const unsigned g = (unsigned)std::max<int64_t>(1, (n + per_tile - 1) / per_tile);
     const bool vec = (uintptr_t)lengths % 16 == 0;
