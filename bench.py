@@ -45,6 +45,8 @@ def parse_args():
     p.add_argument("--batches", type=int, default=None,
                    help="distinct id batches rotated through (default 32 for c2, 12 for c4, 8 elsewhere)")
     p.add_argument("--mode", default="eager", choices=["graph", "eager"])
+    p.add_argument("--split-bags", type=int, default=1,
+                   help="c5 only: cut every bag of 80 into N bags of 80/N (bounds what splitting long bags could gain)")
     p.add_argument("--row-alignment", type=int, default=None, help="default 16 (TorchRec's), 4 for c5 (68-byte rows)")
     p.add_argument("--row-padding", default=None, choices=["line", "none"],
                    help="distance between rows in the packed store: 'line' = rows of at most 128 bytes at the next "
@@ -175,10 +177,19 @@ def build_workload(args, dev):
         T, B = 8, 16384
         rows = [max(1000, int(250_000_000 * args.scale))] * T
         dims, dts = [128] * T, ["int4"] * T
-        lens = lambda: np.full(T * B, 80, dtype=np.int64)
+        # --split-bags N: every bag of 80 cut into N bags of 80 / N (N x the bags, the same ids in the same
+        # order): what a lookup that splits long bags over N lane groups would pool before its
+        # cross-lane reduction, i.e. a lower bound on that variant's time.
+        split = max(1, int(getattr(args, "split_bags", 1) or 1))
+        if 80 % split:
+            raise SystemExit("--split-bags must divide 80")
+        B *= split
+        lens = lambda: np.full(T * B, 80 // split, dtype=np.int64)
         pooling = PoolingType.MEAN
         id_fn = None  # affine bijection below: a 250M-entry permutation per table is not needed
         desc = "c5: QEBC 8 tables x 250M x 128 int4 (68 B rows), B16384, L=80, Zipf(0.8), MEAN, fp16 out"
+        if split > 1:
+            desc += f" [every bag split into {split} bags of {80 // split}: B{B}; not the c5 workload]"
 
     if getattr(args, "batch_size", None):
         B = args.batch_size

@@ -118,7 +118,8 @@ int tra_tbe_destroy(tra_tbe_t tbe);
  * Arithmetic per output column, ids in order: acc = fmaf(w*scale, q, acc +
  * w*bias) (fp16/fp32 rows: acc = fmaf(w, x, acc)); MEAN multiplies by 1.0f/len;
  * output rounded to nearest even.  Ids outside [0, rows) other than -1 are
- * skipped and counted (tra_tbe_error_count).  Every buffer sits at a multiple
+ * counted (tra_tbe_error_count) and skipped, or pool row 0 where
+ * tra_tbe_set_bounds_check_mode asked for that.  Every buffer sits at a multiple
  * of its element size (weights: 4 bytes), else TRA_ERR_INVALID_ARGUMENT. */
 int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
                     const void* offsets, int32_t idx_is_i64,
@@ -207,9 +208,22 @@ int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
                         int32_t pooling_mode, int32_t lengths_num_keys, char* buf,
                         int32_t buf_len);
 
+/* What later forwards on this plan do with an id outside [0, rows) other than
+ * -1, by fbgemm_gpu's BoundsCheckMode codes (the `bounds_check_mode` the
+ * reference hands to the TBE constructor, default WARNING, at
+ * torchrec/distributed/quant_embedding_kernel.py:281-283, 337-339):
+ *   WARNING 1, IGNORE 2   the id pools row 0, as after bounds_check_indices,
+ *                         which rewrites such an id to 0 in these modes
+ *   FATAL 0, NONE 3, -1   the id is skipped (pools nothing); this is a new
+ *                         plan's behaviour.  (The caller raises for FATAL from
+ *                         tra_tbe_error_count; NONE means unchecked in fbgemm.)
+ * Counted by tra_tbe_error_count in every mode.  Calls already launched keep
+ * the mode they were launched with. */
+int tra_tbe_set_bounds_check_mode(tra_tbe_t tbe, int32_t mode);
+
 /* Number of out-of-range ids seen by forwards on this plan since the last
- * call (synchronizes the stream; resets the counter).  Stands in for
- * fbgemm_gpu's bounds_check_indices. */
+ * call (synchronizes the stream; resets the counter).  Stands in for the
+ * report of fbgemm_gpu's bounds_check_indices. */
 int tra_tbe_error_count(tra_tbe_t tbe, void* stream, int64_t* count);
 
 /* Index math -------------------------------------------------------------- */

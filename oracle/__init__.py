@@ -230,6 +230,27 @@ def tbe_forward(
 # --------------------------------------------------------------------------
 # index math
 # --------------------------------------------------------------------------
+def bounds_check_indices(rows_per_feature: Sequence[int], B: int, indices: np.ndarray, offsets: np.ndarray,
+                         mode: str) -> Tuple[np.ndarray, int]:
+    """What fbgemm_gpu's ``bounds_check_indices`` leaves of the ids before the lookup runs: in the
+    WARNING and IGNORE modes an id outside [0, rows) of its feature's table, other than the pruned
+    id -1, is rewritten to 0 (``"NONE"``: ids untouched).  Returns (ids, number of such ids).
+    PARITY UNPINNED: fbgemm_gpu (unpinned dependency of the reference, requirements.txt:4) is not
+    in this image and the reference holds no fixture for out-of-range ids; this restates the
+    operator's documented behaviour at the call site that selects the mode
+    (torchrec/distributed/quant_embedding_kernel.py:337-339).  Offsets are taken as valid."""
+    ids = np.array(indices, copy=True)
+    bad_total = 0
+    for f, rows in enumerate(rows_per_feature):
+        lo, hi = int(offsets[f * B]), int(offsets[(f + 1) * B])
+        seg = ids[lo:hi]
+        bad = ((seg < 0) | (seg >= rows)) & (seg != -1)
+        bad_total += int(bad.sum())
+        if mode in ("WARNING", "IGNORE"):
+            seg[bad] = 0
+    return ids, bad_total
+
+
 def cumsum(lengths: np.ndarray) -> np.ndarray:
     lengths = np.ascontiguousarray(lengths)
     out = np.zeros(lengths.shape[0] + 1, dtype=lengths.dtype)

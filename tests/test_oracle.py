@@ -251,3 +251,20 @@ def test_bucketize_oracle_matches_python_rule(F, B, W, idt, keep):
     # without weights / without the permute the other outputs do not change
     ol2, oi2, ow2, ou2 = O.bucketize(lengths, ids, block_sizes, W, None, keep)
     assert ol2.tolist() == pl and oi2.tolist() == pi and ow2 is None and ou2 is None
+
+
+def test_bounds_check_oracle_hand_case():
+    """The restated id rewrite of fbgemm_gpu's bounds_check_indices on a case worked by hand: three
+    features x two bags; -1 stays, every other id outside its own feature's table becomes 0 in
+    WARNING / IGNORE and stays in NONE; an id that is fine for a larger table is bad for a smaller
+    one.  (Unpinned against fbgemm_gpu itself, which this image does not have.)"""
+    rows = [4, 10, 6]
+    offsets = np.array([0, 2, 3, 6, 6, 8, 9])
+    ids = np.array([3, 4, -1, 9, 10, -7, 5, 6, 0])
+    #               f0    | f0 | f1        | f1 (empty) | f2   | f2
+    for mode in ("WARNING", "IGNORE"):
+        out, bad = O.bounds_check_indices(rows, 2, ids, offsets, mode)
+        assert out.tolist() == [3, 0, -1, 9, 0, 0, 5, 0, 0] and bad == 4
+    out, bad = O.bounds_check_indices(rows, 2, ids, offsets, "NONE")
+    assert out.tolist() == ids.tolist() and bad == 4
+    assert ids.tolist() == [3, 4, -1, 9, 10, -7, 5, 6, 0]  # the input is not modified

@@ -23,7 +23,7 @@ ST = {O.FP32: SparseType.FP32, O.FP16: SparseType.FP16, O.INT8: SparseType.INT8,
 POOL = {O.SUM: PoolingMode.SUM, O.MEAN: PoolingMode.MEAN, O.NONE: PoolingMode.NONE}
 
 
-def build(rng, specs, ftm, pooling, out_dtype, row_alignment, row_padding=None):
+def build(rng, specs, ftm, pooling, out_dtype, row_alignment, row_padding=None, bounds_check_mode=None):
     """specs: [(dtype, rows, dim)].  Returns (TBE on GPU, oracle Store).  The packed store's row
     padding (rows of up to 128 bytes at a power-of-two stride, or every row at its width) is drawn
     from the test's generator unless given: the oracle has its own copy of the tables, so the
@@ -41,6 +41,7 @@ def build(rng, specs, ftm, pooling, out_dtype, row_alignment, row_padding=None):
         embedding_specs=[(f"t{i}", rows, dim, ST[dt], EmbeddingLocation.DEVICE) for i, (dt, rows, dim) in enumerate(specs)],
         feature_table_map=ftm, pooling_mode=POOL[pooling], device=DEV, weight_lists=weight_lists,
         output_dtype=ST[out_dtype], row_alignment=row_alignment, row_padding=row_padding,
+        bounds_check_mode=bounds_check_mode,
     )
     return tbe, store
 
@@ -1035,3 +1036,64 @@ def test_table_beyond_2_31_rows(tuning):
     assert tbe.out_of_range_count() == 0
     del tbe, w
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("mode", ["WARNING", "IGNORE"])
+def test_bounds_check_warning_and_ignore_pool_row_zero(mode, tuning):
+    """BoundsCheckMode.WARNING / IGNORE: an id outside its table (too large, or negative other than
+    -1) pools row 0 of that table, which is what the lookup sees in fbgemm_gpu after
+    bounds_check_indices has rewritten the id to 0 (the reference's sharded call site asks for
+    WARNING by default, torchrec/distributed/quant_embedding_kernel.py:337-339); -1 is still
+    skipped; every bad id is counted.  Parity unpinned: fbgemm_gpu is not in this image, the
+    expectation is its documented behaviour restated on the oracle (bad ids replaced by 0).
+    Covered: both pooled kernels, ids a block at a time (8 lanes per row) and one by one, per-sample
+    weights, MEAN, both id widths, the lookup from lengths, and the sequence lookup."""
+    from torchrec_amd.tbe.enums import BoundsCheckMode
+    bcm = getattr(BoundsCheckMode, mode)
+    rng = np.random.default_rng(77 + len(mode))
+    for (dt, dim), pooling, weighted, idt, balanced in itertools.product(
+        ((O.INT4, 128), (O.INT8, 32), (O.FP16, 64), (O.INT2, 256)), (O.SUM, O.MEAN), (False, True),
+        (np.int32, np.int64), (0, 1),
+    ):
+        rows, B = 500, 70
+        specs = [(dt, rows, dim), (dt, rows + 40, dim)]
+        ftm = [0, 1, 1]
+        rows_f = [rows, rows + 40, rows + 40]
+        tbe, store = build(rng, specs, ftm, pooling, O.FP32, 16, bounds_check_mode=bcm)
+        tuning(balanced=balanced)
+        lengths, offsets, ids = make_bags(rng, rows_f, B, 45, idt)
+        feat_of = np.repeat(np.arange(3), B)
+        owner = np.repeat(feat_of, lengths)  # feature of every id
+        bad = ids.copy()
+        pick = rng.choice(len(ids), 60, replace=False)
+        bad[pick[:20]] = -1                                              # pruned: skipped, not counted
+        bad[pick[20:40]] = np.asarray(rows_f)[owner[pick[20:40]]] + rng.integers(0, 5, 20)  # too large
+        bad[pick[40:]] = -2 - rng.integers(0, 1000, 20)                   # negative, not -1
+        expect, n_bad = O.bounds_check_indices(rows_f, B, bad, offsets, mode)
+        assert n_bad == 40 and (expect[pick[20:]] == 0).all() and (expect[pick[:20]] == -1).all()
+        psw = rng.uniform(-1, 1, len(ids)).astype(np.float32) if weighted else None
+        tag = (dt, dim, pooling, weighted, idt, balanced)
+        want = O.tbe_forward(store, ftm, B, expect, offsets, psw, pooling, O.FP32)
+        got = tbe(torch.from_numpy(bad).to(DEV), torch.from_numpy(offsets).to(DEV),
+                  None if psw is None else torch.from_numpy(psw).to(DEV)).cpu().numpy()
+        assert bits_equal(got, want) == 0, tag
+        assert tbe.out_of_range_count() == 40, tag
+        if not weighted:
+            # the same from the lengths (the collection's route)
+            got = tbe(torch.from_numpy(bad).to(DEV), None, None, lengths=torch.from_numpy(lengths.astype(idt)).to(DEV),
+                      batch_size=B).cpu().numpy()
+            assert bits_equal(got, want) == 0, tag
+            assert tbe.out_of_range_count() == 40, tag
+    # sequence lookup: the row of a bad id is row 0 of its table, that of -1 is zeros
+    rows, dim, B = 300, 64, 9
+    tbe, store = build(rng, [(O.INT8, rows, dim), (O.INT8, rows, dim)], [0, 1], O.NONE, O.FP16, 16, bounds_check_mode=bcm)
+    lengths, offsets, ids = make_bags(rng, [rows, rows], B, 12, np.int32)
+    bad = ids.copy()
+    bad[::5] = rows + 1
+    bad[1::7] = -1
+    expect, n_bad = O.bounds_check_indices([rows, rows], B, bad, offsets, mode)
+    assert n_bad == int((bad == rows + 1).sum())
+    want = O.tbe_forward(store, [0, 1], B, expect, offsets, None, O.NONE, O.FP16)
+    got = tbe(torch.from_numpy(bad).to(DEV), torch.from_numpy(offsets).to(DEV)).cpu().numpy()
+    assert bits_equal(got, want) == 0
+    assert tbe.out_of_range_count() == int((bad == rows + 1).sum())

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = [
     "tra_tbe_forward_lengths_static",
     "tra_tbe_forward_position_weighted",
     "tra_tbe_launch_info",
+    "tra_tbe_set_bounds_check_mode",
     "tra_tbe_error_count",
     "tra_cumsum_workspace_bytes",
     "tra_cumsum",
@@ -101,6 +102,7 @@ def lib() -> ctypes.CDLL:
             vp, i64, vp, vp,
         ]
         l.tra_tbe_launch_info.argtypes = [vp, i32, i64, i32, i32, ctypes.c_char_p, i32]
+        l.tra_tbe_set_bounds_check_mode.argtypes = [vp, i32]
         l.tra_tbe_error_count.argtypes = [vp, vp, ctypes.POINTER(i64)]
         l.tra_cumsum_workspace_bytes.argtypes = [i64]
         l.tra_cumsum_workspace_bytes.restype = i64

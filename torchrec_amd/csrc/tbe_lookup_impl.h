@@ -56,6 +56,7 @@ struct LookupArgs {
   int32_t mean;
   int32_t vec_store;  // 1: every lane's output slice is 16-byte aligned
   int32_t out_fp16;
+  int32_t bad_to_row0;  // 1: an id outside its table (other than -1) reads row 0 instead of being skipped
   int32_t xcd_blocks;   // balanced pooled kernel: blocks per XCD (0: no XCD remap)
   int32_t xcd_count;    // balanced pooled kernel: XCDs the grid is dealt to
   int16_t feat_pos[kMaxPos];  // balanced pooled kernel: key position of the class's first features
@@ -504,7 +505,7 @@ __device__ __forceinline__ bool locate_tile(const LookupArgs& a, int& f, int& lp
 // U rows ahead, row chunks one batch ahead, so neither an id load nor a row
 // load is waited for in the batch that issued it.
 template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, int NE>
-__device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
+__device__ __forceinline__ int pool_bag(float (&acc)[NE], const LookupArgs& a,
                                          const RowWalk& w, int64_t start64, int len,
                                          int max_len_any_lane) {
   // Wave-uniform by construction; telling the compiler keeps the loop control
@@ -547,6 +548,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
   }
   // Bad ids are counted by the lane that owns column 0.
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
+  return bad;
 }
 
 // The same pooling with the ids fetched a whole lane group at a time: lane c of
@@ -562,7 +564,7 @@ __device__ __forceinline__ void pool_bag(float (&acc)[NE], const LookupArgs& a,
 // conditional load it has to assume the worst and drains all loads, which
 // undoes the double buffering once per iteration.)
 template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int U, int NE, bool TWO_BATCHES = false>
-__device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs& a,
+__device__ __forceinline__ int pool_bag_bulk(float (&acc)[NE], const LookupArgs& a,
                                               const RowWalk& w, int64_t start64, int len,
                                               int max_len_any_lane, int lpr, int c,
                                               int group_lane0) {
@@ -676,6 +678,32 @@ __device__ __forceinline__ void pool_bag_bulk(float (&acc)[NE], const LookupArgs
       if (it + U + u < max_len) consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, bufB[u], w);
   }
   if (bad != 0 && w.count_errors) atomicAdd(a.err_count, (unsigned long long)bad);
+  return bad;
+}
+
+// The bags of a wave pooled once more, where the launch wants an id outside
+// its table to pool row 0 (what fbgemm's bounds_check_indices makes of such an
+// id in its WARNING and IGNORE modes: it rewrites it to 0) and one of the
+// wave's bags held such an id.  The pooling loops above skip it; since the
+// order of the additions is part of the result, the bag cannot be corrected
+// afterwards and is pooled again from zero, one row at a time (rare by
+// assumption: bad ids are an input error).  Bad ids are not counted again.
+template <int DTYPE, int CB, typename IdxT, int WEIGHTED, int NE>
+__device__ __forceinline__ void repool_bad_ids_as_row0(float (&acc)[NE], const LookupArgs& a,
+                                                    const RowWalk& w, int64_t start64, int len,
+                                                    int max_len_any_lane) {
+  const int max_len = __builtin_amdgcn_readfirstlane(max_len_any_lane);
+  const IdxT start = (IdxT)start64;
+  const IdxT last = (IdxT)(a.num_indices - 1);
+#pragma unroll
+  for (int k = 0; k < NE; ++k) acc[k] = 0.0f;
+  for (int r = 0; r < max_len; ++r) {
+    const IdxT id = fetch_id<IdxT>(a, r < len, start + (IdxT)r, last);
+    RowBuf<CB> buf;
+    fetch_row<DTYPE, CB, WEIGHTED, IdxT>(buf, id, start + (IdxT)r, last, a, w);
+    if (id != (IdxT)-1) buf.valid = 1;  // fetch_row has redirected an id outside the table to row 0
+    consume_row<DTYPE, CB, (WEIGHTED != 0)>(acc, buf, w);
+  }
 }
 
 // Finish one bag per lane group (MEAN scaling, rounding, store).  Lane c of the
@@ -1045,7 +1073,9 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
   float acc[NE];
 #pragma unroll
   for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
-  pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+  const int bad = pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+  if (a.bad_to_row0 != 0 && __builtin_amdgcn_ballot_w64(bad != 0) != 0)
+    repool_bad_ids_as_row0<DTYPE, CB, IdxT, WEIGHTED, NE>(acc, a, w, start, len, max_len);
   TRA_STAMP(2);
 #ifdef TRA_INSTRUMENT
   if ((threadIdx.x & 63) == 0)
@@ -1396,13 +1426,16 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(
     float acc[NE];
 #pragma unroll
     for (int k = 0; k < NE; ++k) acc[k] = 0.0f;
+    int bad;
     if (U == 4 && lpr >= 2 * U && (lpr & (lpr - 1)) == 0)
       if (lpr == 2 * U)
-        pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE, true>(acc, a, w, start, len, max_len, lpr, c, lane - c);
+        bad = pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE, true>(acc, a, w, start, len, max_len, lpr, c, lane - c);
       else
-        pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len, lpr, c, lane - c);
+        bad = pool_bag_bulk<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len, lpr, c, lane - c);
     else
-      pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+      bad = pool_bag<DTYPE, CB, IdxT, WEIGHTED, U, NE>(acc, a, w, start, len, max_len);
+    if (a.bad_to_row0 != 0 && __builtin_amdgcn_ballot_w64(bad != 0) != 0)
+      repool_bad_ids_as_row0<DTYPE, CB, IdxT, WEIGHTED, NE>(acc, a, w, start, len, max_len);
     TRA_STAMP(3);
 #ifdef TRA_INSTRUMENT
     if (lane == 0) a.ts[((size_t)blockIdx.x * (blockDim.x / 64) + wave) * 8 + 5] = (unsigned long long)max_len;
@@ -1450,6 +1483,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
     const IdxT id = reinterpret_cast<const IdxT*>(a.indices)[j];
     const int bad = fetch_row<DTYPE, CB, false, IdxT>(r, id, (IdxT)j, (IdxT)(a.num_indices - 1), a, w);
     if (bad && w.count_errors) atomicAdd(a.err_count, 1ull);
+    if (bad && a.bad_to_row0 != 0) r.valid = 1;  // the row fetched for it is row 0
     float acc[NE];
 #pragma unroll
     for (int i = 0; i < NE; ++i) acc[i] = 0.0f;

@@ -186,6 +186,7 @@ struct tra_tbe {
   FeatureDesc* cdescs_dev = nullptr;  // the descriptors in that order: cdescs[i] = slices[feats[i]]
   unsigned long long* err_dev = nullptr;
   void* static_scratch = nullptr;  // this device's copy of the library's static scratch array
+  std::atomic<int> bad_to_row0{0};  // 1: ids outside their table pool row 0 (tra_tbe_set_bounds_check_mode)
   std::vector<LaunchClass> classes;
   std::vector<LookupArgs> base_args;  // per class: everything a call does not change
   std::mutex geo_mutex;
@@ -297,8 +298,9 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     // the all-64-byte one).
     int cb = payload % 16 == 0 && payload > 64 ? 16 : (payload % 8 == 0 ? 8 : 4);
     {
-      const int force = g_ovr.cb;  // tuning: smaller lane chunks
+      const int force = g_ovr.cb;  // tuning: smaller lane chunks, or 16 bytes wherever they divide the row
       if ((force == 8 || force == 4) && force < cb && payload % force == 0) cb = force;
+      if (force == 16 && payload % 16 == 0) cb = 16;
     }
     const int max_slice = cb * kWaveSize;  // bytes one wave-wide lane group covers
     // A row with a header whose lanes take 8 or 4 bytes normally gets its header with the
@@ -760,6 +762,7 @@ static int forward_impl(tra_tbe_t tbe, const void* weights, const void* indices,
     }
     a.out = out;
     a.out_stride = out_stride;
+    a.bad_to_row0 = tbe->bad_to_row0.load(std::memory_order_relaxed);
     a.num_indices = num_indices > 0 ? num_indices : 1;
     a.B = batch_size;
     a.mean = pooling_mode == TRA_POOL_MEAN;
@@ -927,6 +930,19 @@ int tra_tbe_forward_position_weighted(tra_tbe_t tbe, const void* weights, const 
                                 workspace, stream, &pw);
   return forward_impl(tbe, weights, indices, bags, false, idx_is_i64, nullptr, batch_size,
                       num_indices, pooling_mode, out_dtype, out, out_stride, stream, &pw);
+}
+
+int tra_tbe_set_bounds_check_mode(tra_tbe_t tbe, int32_t mode) {
+  if (!tbe) {
+    set_error("tra_tbe_set_bounds_check_mode: null plan");
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  if (mode < -1 || mode > 3) {
+    set_error("tra_tbe_set_bounds_check_mode: mode %d is none of FATAL 0, WARNING 1, IGNORE 2, NONE 3, unset -1", mode);
+    return TRA_ERR_INVALID_ARGUMENT;
+  }
+  tbe->bad_to_row0.store(mode == 1 || mode == 2 ? 1 : 0, std::memory_order_relaxed);
+  return TRA_OK;
 }
 
 int tra_tbe_error_count(tra_tbe_t tbe, void* stream, int64_t* count) {

@@ -135,9 +135,11 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
         self.embedding_specs = embedding_specs
         self.pooling_mode = pooling_mode
         self.output_dtype: int = output_dtype.as_int()
-        # An id outside [0, rows) is skipped (adds nothing) and counted in every
-        # mode; BoundsCheckMode.FATAL also raises after the call, which waits
-        # for the kernel.
+        # An id outside [0, rows) is counted in every mode.  WARNING / IGNORE: it
+        # pools row 0, as in fbgemm_gpu, whose bounds_check_indices rewrites such
+        # an id to 0 in these modes before the lookup.  Not given, NONE (unchecked
+        # in fbgemm_gpu) and FATAL: it is skipped (adds nothing); FATAL also raises
+        # after the call, which waits for the kernel.
         self.bounds_check_mode_int: int = -1 if bounds_check_mode is None else int(bounds_check_mode)
         if output_dtype not in (SparseType.FP32, SparseType.FP16):
             raise NotImplementedError(f"output dtype {output_dtype} (fp32 and fp16 are supported)")
@@ -358,6 +360,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(nn.Module):
             plan = ctypes.c_void_p()
             with torch.cuda.device(self.current_device):
                 _lib.check(_lib.lib().tra_tbe_create(specs, T_, ftm, pos, F, ctypes.byref(plan)))
+            if self.bounds_check_mode_int >= 0:
+                _lib.check(_lib.lib().tra_tbe_set_bounds_check_mode(plan, self.bounds_check_mode_int))
             self._plans[feature_positions] = plan
         return plan
 
