@@ -72,7 +72,9 @@ int tra_device_arch(char* buf, int buf_len);
  * window kernel, 0: static kernel), "window" (bags per block), "unroll", "lds",
  * "xcd" (0: no remap of blocks to dies), "cost_floor", "fused_scan" (from-lengths
  * prologue inside the lookup kernel: 1 always, 0 never), "cb" (lane chunk bytes,
- * acts on plans created afterwards); value < 0 restores the default.  The
+ * acts on plans created afterwards), "fork" (0: the launches of a call of three
+ * or more launch classes all stay on the caller's stream instead of alternating
+ * with the plan's second stream); value < 0 restores the default.  The
  * same knobs are read from the environment (TRA_BALANCED, TRA_WINDOW, ...)
  * once, when the library is loaded; no lookup call reads the environment.
  * Process-wide; not meant to be changed while lookups are being issued.
@@ -120,7 +122,12 @@ int tra_tbe_destroy(tra_tbe_t tbe);
  * output rounded to nearest even.  Ids outside [0, rows) other than -1 are
  * counted (tra_tbe_error_count) and skipped, or pool row 0 where
  * tra_tbe_set_bounds_check_mode asked for that.  Every buffer sits at a multiple
- * of its element size (weights: 4 bytes), else TRA_ERR_INVALID_ARGUMENT. */
+ * of its element size (weights: 4 bytes), else TRA_ERR_INVALID_ARGUMENT.
+ * Ordering: everything the call launches runs after what `stream` holds at the
+ * call and before what is put on `stream` afterwards.  A plan of three or more
+ * launch classes (weight type x lane chunk) runs every other launch on a second
+ * stream of its own, forked from and joined to `stream` with events inside the
+ * call; not while `stream` is being captured into a graph. */
 int tra_tbe_forward(tra_tbe_t tbe, const void* weights, const void* indices,
                     const void* offsets, int32_t idx_is_i64,
                     const float* per_sample_weights, int32_t batch_size,

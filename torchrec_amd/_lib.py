@@ -154,7 +154,7 @@ def check(rc: int) -> None:
 
 def set_tuning(**knobs: Optional[int]) -> None:
     """Tuning overrides of the lookup (``balanced``, ``window``, ``unroll``, ``lds``, ``xcd``,
-    ``cost_floor``, ``fused_scan``, ``cb``); ``None`` restores a knob's default.  For
+    ``cost_floor``, ``fused_scan``, ``cb``, ``fork``); ``None`` restores a knob's default.  For
     experiments and tests: process-wide, and not to be changed while lookups are in flight."""
     for name, value in knobs.items():
         check(lib().tra_set_tuning(name.encode(), -1 if value is None else int(value)))
