@@ -14,7 +14,7 @@ kernel (``tra_copy_bytes``, 256 MiB, timed in the same run) reaches.  A call
 that consists of several launches (permute, bucketize) is timed as a whole; the
 per-kernel durations are in the rocprofv3 summaries under ``profiles/``.
 
-Shapes (BASELINE.json configs): c2 = 26 features x B 2048, lengths U[1,40] with
+Shapes (the benchmark configurations): c2 = 26 features x B 2048, lengths U[1,40] with
 5 % empty; c3 = 64 x 4096, Poisson(30); c5 = 8 x 16384, fixed 80.
 """
 from __future__ import annotations

@@ -203,8 +203,10 @@ int tra_tbe_forward_position_weighted(tra_tbe_t tbe, const void* weights, const 
                                       int64_t out_stride, void* workspace, void* stream);
 
 /* Which kernels a tra_tbe_forward with these sizes launches, one entry per
- * launch, "; "-separated, e.g. "tbe_pooled_cu_kernel dtype=int4 lane_bytes=8
- * slices=26".  lengths_num_keys > 0 asks about tra_tbe_forward_lengths with
+ * launch in launch order, "; "-separated, e.g. "tbe_pooled_cu_kernel dtype=int4
+ * lane_bytes=8 slices=26"; where the launches alternate between two streams
+ * an entry also says which ("... on the plan's second stream").
+ * lengths_num_keys > 0 asks about tra_tbe_forward_lengths with
  * that many keys instead (entries then end in " from_lengths" when the kernel
  * derives the offsets itself, else the scan kernels come first).  For
  * profiling: the names are the ones a kernel trace shows.

@@ -555,12 +555,17 @@ int tra_tbe_launch_info(tra_tbe_t tbe, int32_t batch_size, int64_t num_indices,
                                                 (const void*)16));
   static const char* const kDtypeName[] = {"fp32", "fp16", "int8", "int4", "int2"};
   std::string text;
-  for (const LaunchClass& cls : tbe->classes) {
-    char line[160];
-    snprintf(line, sizeof(line), "%s%s dtype=%s lane_bytes=%d slices=%d%s",
+  // In launch order; a plan with a second stream alternates between the two.
+  const bool two_streams = tbe->side != nullptr && balanced && g_ovr.fork != 0;
+  for (const int ci : tbe->launch_order) {
+    const LaunchClass& cls = tbe->classes[ci];
+    char line[200];
+    snprintf(line, sizeof(line), "%s%s dtype=%s lane_bytes=%d slices=%d%s%s",
              text.empty() ? "" : "; ",
              nobag ? "tbe_nobag_kernel" : (balanced ? "tbe_pooled_cu_kernel" : "tbe_pooled_kernel"),
-             kDtypeName[cls.dtype], cls.cb, (int)cls.feats.size(), fused ? " from_lengths" : "");
+             kDtypeName[cls.dtype], cls.cb, (int)cls.feats.size(),
+             two_streams ? (tbe->on_side[ci] ? " on the plan's second stream" : " on the caller's stream") : "",
+             fused ? " from_lengths" : "");
     text += line;
   }
   if (lengths_num_keys > 0 && !fused) text = "scan_small_kernel or tile_sums_kernel + scan_tiles_kernel; " + text;

@@ -460,34 +460,41 @@ class EmbeddingBagCollection(EmbeddingBagCollectionInterface, ModuleNoCopyMixin,
         ):
             op = ops_[0]
             v, ln, keys = features._values, features._lengths, features._keys
+            # (devices are compared by index: get_device() is -1 for a host tensor, and the
+            # operator's device always carries an index)
+            dev = op.current_device
+            di = dev.index if dev.type == "cuda" else -2
+            vdt = v.dtype
             if (
                 ln is not None
                 and (keys is self._feature_names or keys == self._feature_names)
-                and v.is_cuda
-                and ln.is_cuda
-                and (v.dtype is torch.int64 or v.dtype is torch.int32)
-                and ln.dtype is v.dtype
-                and ln.device == v.device
+                and v.get_device() == di
+                and ln.get_device() == di
+                and (vdt is torch.int64 or vdt is torch.int32)
+                and ln.dtype is vdt
                 and ln.dim() == 1
                 and v.is_contiguous()
                 and ln.is_contiguous()
                 and op._weights_initialized
-                and v.device == op.current_device
-                and op._buffers["weights_dev"].device == v.device
+                and op._buffers["weights_dev"].get_device() == di
                 and not getattr(self, MODULE_ATTR_CACHE_FEATURES_ORDER, False)
             ):
                 K = len(keys)
-                B = ln.numel() // K if K else 0
+                n_len = ln.numel()
+                B = n_len // K if K else 0
                 # (a feature that feeds two tables appears twice among the module's feature names: its
                 # bags are then read twice from one key, which the general route below resolves)
+                unique = self.__dict__.get("_feature_names_are_unique")
+                if unique is None:
+                    unique = self._feature_names_unique()
                 if (
                     B > 0
-                    and ln.numel() == K * B
+                    and n_len == K * B
                     and features._stride in (None, B)
                     and features._stride_per_key is None
-                    and self._feature_names_unique()
+                    and unique
                 ):
-                    out = torch.empty(B, self._total_D, dtype=self._output_dtype, device=v.device)
+                    out = torch.empty(B, self._total_D, dtype=self._output_dtype, device=dev)
                     op._launch_from_lengths(
                         None, v, ln, int(v.dtype is torch.int64), None, B, K, v.numel(), out.data_ptr(), out.stride(0)
                     )
