@@ -72,9 +72,10 @@ int tra_device_arch(char* buf, int buf_len);
  * window kernel, 0: static kernel), "window" (bags per block), "unroll", "lds",
  * "xcd" (0: no remap of blocks to dies), "cost_floor", "fused_scan" (from-lengths
  * prologue inside the lookup kernel: 1 always, 0 never), "cb" (lane chunk bytes,
- * acts on plans created afterwards), "fork" (0: the launches of a call of three
+ * acts on plans created afterwards), "fork" (0: the launches of a call of five
  * or more launch classes all stay on the caller's stream instead of alternating
- * with the plan's second stream); value < 0 restores the default.  The
+ * with the plan's second stream; k > 1, for plans created afterwards: from k
+ * classes on instead of five); value < 0 restores the default.  The
  * same knobs are read from the environment (TRA_BALANCED, TRA_WINDOW, ...)
  * once, when the library is loaded; no lookup call reads the environment.
  * Process-wide; not meant to be changed while lookups are being issued.
@@ -124,7 +125,7 @@ int tra_tbe_destroy(tra_tbe_t tbe);
  * tra_tbe_set_bounds_check_mode asked for that.  Every buffer sits at a multiple
  * of its element size (weights: 4 bytes), else TRA_ERR_INVALID_ARGUMENT.
  * Ordering: everything the call launches runs after what `stream` holds at the
- * call and before what is put on `stream` afterwards.  A plan of three or more
+ * call and before what is put on `stream` afterwards.  A plan of five or more
  * launch classes (weight type x lane chunk) runs every other launch on a second
  * stream of its own, forked from and joined to `stream` with events inside the
  * call; not while `stream` is being captured into a graph. */

@@ -1100,7 +1100,7 @@ def test_bounds_check_warning_and_ignore_pool_row_zero(mode, tuning):
 
 
 def test_multi_class_call_on_two_streams(tuning):
-    """A plan of three or more launch classes runs every other launch on its own second stream,
+    """A plan of five or more launch classes runs every other launch on its own second stream,
     forked from and joined to the caller's stream inside the call.  Checked: the same bits as with
     everything on the caller's stream (tuning fork=0) and as the oracle on a sample of bags; the call
     is ordered behind work queued on the caller's stream before it (inputs written by a kernel just
@@ -1121,10 +1121,21 @@ def test_multi_class_call_on_two_streams(tuning):
     n = int(offsets[-1])
     batches = [rng.integers(0, rows, n).astype(np.int32) for _ in range(4)]
     to = torch.from_numpy(offsets).to(DEV)
+    import ctypes
+    from torchrec_amd import _lib
+
+    def launches():
+        buf = ctypes.create_string_buffer(4096)
+        _lib.check(_lib.lib().tra_tbe_launch_info(tbe._get_plan(None), B, n, int(tbe.pooling_mode), 0, buf, 4096))
+        return buf.value.decode().split("; ")
+
     tuning(fork=0)
+    assert len(launches()) == 7 and not any("stream" in x for x in launches())
     want = [tbe(torch.from_numpy(b).to(DEV), to).clone() for b in batches]
     torch.cuda.synchronize()
     tuning(fork=None)
+    # seven launch classes: every other launch, largest class first, goes to the second stream
+    assert [("second stream" in x) for x in launches()] == [False, True, False, True, False, True, False], launches()
     # ordering on the caller's stream: ids copied in just before the call, output summed right after
     ti = torch.empty(n, dtype=torch.int32, device=DEV)
     for k in (0, 1, 2, 3, 0):

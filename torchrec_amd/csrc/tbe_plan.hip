@@ -173,8 +173,11 @@ struct Geometry {
 
 constexpr int kGeometrySlots = 8;
 
-// A call of at least this many launch classes runs them on two streams (see forward_impl).
-constexpr size_t kForkMinClasses = 3;
+// A call of at least this many launch classes runs them on two streams (see forward_impl).  The
+// fork and the join cost about 10 us of dependencies between queues, every pair of neighbouring
+// launches gains a few: with launches of 25 - 30 us each, two classes lose 11 %, three and four
+// are even (-1 %, +0.5 %), five gain 8 %, seven (of about 50 us) 9 %.
+constexpr size_t kForkMinClasses = 5;
 
 struct tra_tbe {
   int device = 0;
@@ -192,7 +195,7 @@ struct tra_tbe {
   unsigned long long* err_dev = nullptr;
   void* static_scratch = nullptr;  // this device's copy of the library's static scratch array
   std::atomic<int> bad_to_row0{0};  // 1: ids outside their table pool row 0 (tra_tbe_set_bounds_check_mode)
-  // The second stream of a multi-class call (plans of kForkMinClasses classes or more; default
+  // The second stream of a multi-class call (plans of kForkMinClasses launch classes or more; default
   // priority), the events that fork it from and join it to the caller's stream, and which of the
   // two streams every class is launched on, in launch order (largest class first).
   std::mutex fork_mutex;
@@ -462,7 +465,9 @@ int tra_tbe_create(const tra_table_spec* tables, int32_t num_tables,
     plan->launch_order.resize(nc);
     for (size_t ci = 0; ci < nc; ++ci) plan->launch_order[ci] = (int)ci;
     plan->on_side.assign(nc, 0);
-    if (nc >= kForkMinClasses) {
+    // (tuning: `fork` = k > 1 at plan creation lowers or raises the class count from which a plan forks)
+    const size_t fork_min = g_ovr.fork > 1 ? (size_t)g_ovr.fork : kForkMinClasses;
+    if (nc >= fork_min) {
       std::stable_sort(plan->launch_order.begin(), plan->launch_order.end(),
                        [&](int x, int y) { return cost[x] > cost[y]; });
       for (size_t k = 0; k < nc; ++k) plan->on_side[plan->launch_order[k]] = (uint8_t)(k & 1);
