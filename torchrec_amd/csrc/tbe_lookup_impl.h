@@ -163,23 +163,57 @@ __device__ __forceinline__ void fma_step(float& acc, float s, float q, float b) 
   acc = __builtin_fmaf(s, q, t);
 }
 
+// Sub-byte fields to floats on the matrix core.  Eight bytes 0x00 .. 0x0f per
+// lane (two payload dwords' worth of masked fields) become eight floats with
+// two v_mfma_f32_16x16x32_bf8_fp8: the lane's bytes are one column slice of the
+// B operand (FP8 E4M3: a byte 0x0q is exactly q * 2^-9, subnormals and the
+// first binade), the A operand holds 2^9 (BF8 0x60) where row m selects byte
+// (m & 3) [+ 4] of lane group m >> 2, and C is zero; so output register r of a
+// lane is 2^9 * (its own byte r [+ 4]) plus exact zeros: the integer q, with no
+// rounding anywhere.  This takes the conversions (one v_cvt_pk_f32_fp8 per two
+// elements otherwise) off the vector ALU, which the pooling loop saturates;
+// the matrix core runs beside it.
+typedef float float4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ long mfma_byte_selector(int lane, int half) {
+  const int m = lane & 15, gp = lane >> 4;
+  unsigned long long v = 0;
+  if (gp == (m >> 2)) v = 0x60ull << (8 * ((m & 3) + 4 * half));
+  return (long)v;
+}
+
 // Accumulate the elements of one payload dword.  `acc` points at the
-// accumulators of this dword's elements.  For the unweighted int4/int2 forms
-// the sub-byte fields are converted in place (value q * 2^shift) and the scale
-// is pre-divided by the same power of two: the product is the same real
-// number, so the fused multiply-add rounds identically.  With per-sample
-// weights the scale w*scale may be subnormal, where that division is inexact,
-// so the fields are shifted down instead.
-template <int DTYPE_CODE, bool WEIGHTED>
+// accumulators of this dword's elements.  int4 / int2 fields are converted on
+// the matrix core (mfma_byte_selector above; sel0 / sel1 are the lane's two
+// selector operands), int8 bytes by v_cvt_f32_ubyteN.
+template <int DTYPE_CODE, bool WEIGHTED, bool MATRIX>
 __device__ __forceinline__ void accumulate_dword(float* acc, uint32_t x, float s,
-                                                 float b) {
+                                                 float b, long sel0, long sel1) {
   constexpr int DTYPE = base_type(DTYPE_CODE);
-  if constexpr (DTYPE == TRA_INT8) {
+  if constexpr (DTYPE == TRA_INT4 && MATRIX) {
+    // Low nibbles in the low dword, high nibbles in the high dword of the
+    // matrix instruction's 8-byte operand; element 2k is byte k's low nibble.
+    const uint32_t lo = x & 0x0f0f0f0fu;
+    const uint32_t hi = (x >> 4) & 0x0f0f0f0fu;
+    const long data = (long)(((unsigned long long)hi << 32) | lo);
+    const float4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+    const float4_t l = __builtin_amdgcn_mfma_f32_16x16x32_bf8_fp8(sel0, data, z, 0, 0, 0);
+    const float4_t h = __builtin_amdgcn_mfma_f32_16x16x32_bf8_fp8(sel1, data, z, 0, 0, 0);
+    fma_step(acc[0], s, l[0], b);
+    fma_step(acc[1], s, h[0], b);
+    fma_step(acc[2], s, l[1], b);
+    fma_step(acc[3], s, h[1], b);
+    fma_step(acc[4], s, l[2], b);
+    fma_step(acc[5], s, h[2], b);
+    fma_step(acc[6], s, l[3], b);
+    fma_step(acc[7], s, h[3], b);
+  } else if constexpr (DTYPE == TRA_INT8) {
     fma_step(acc[0], s, byte_to_float<0>(x), b);
     fma_step(acc[1], s, byte_to_float<1>(x), b);
     fma_step(acc[2], s, byte_to_float<2>(x), b);
     fma_step(acc[3], s, byte_to_float<3>(x), b);
   } else if constexpr (DTYPE == TRA_INT4 && !WEIGHTED) {
+    // (16-byte lane chunks: 32 accumulators per lane leave no registers for the
+    // matrix instruction's operands and results, so the vector ALU converts.)
     // A byte 0x0q read as an FP8 (E4M3) value is exactly q * 2^-9 for q = 0..15
     // (subnormals, then the first binade), and one instruction converts two
     // bytes.  The scale is multiplied by 2^9 instead (exact: s is at most
@@ -200,17 +234,35 @@ __device__ __forceinline__ void accumulate_dword(float* acc, uint32_t x, float s
     fma_step(acc[6], s9, l23.y, b);
     fma_step(acc[7], s9, h23.y, b);
   } else if constexpr (DTYPE == TRA_INT4) {
+    // With per-sample weights the scale w*scale may be subnormal, where a
+    // multiplication by 2^9 is inexact, so the fields are shifted down instead.
     const uint32_t lo = x & 0x0f0f0f0fu;
-    const uint32_t hi = WEIGHTED ? ((x >> 4) & 0x0f0f0f0fu) : (x & 0xf0f0f0f0u);
-    const float sh = WEIGHTED ? s : s * 0.0625f;
+    const uint32_t hi = (x >> 4) & 0x0f0f0f0fu;
     fma_step(acc[0], s, byte_to_float<0>(lo), b);
-    fma_step(acc[1], sh, byte_to_float<0>(hi), b);
+    fma_step(acc[1], s, byte_to_float<0>(hi), b);
     fma_step(acc[2], s, byte_to_float<1>(lo), b);
-    fma_step(acc[3], sh, byte_to_float<1>(hi), b);
+    fma_step(acc[3], s, byte_to_float<1>(hi), b);
     fma_step(acc[4], s, byte_to_float<2>(lo), b);
-    fma_step(acc[5], sh, byte_to_float<2>(hi), b);
+    fma_step(acc[5], s, byte_to_float<2>(hi), b);
     fma_step(acc[6], s, byte_to_float<3>(lo), b);
-    fma_step(acc[7], sh, byte_to_float<3>(hi), b);
+    fma_step(acc[7], s, byte_to_float<3>(hi), b);
+  } else if constexpr (DTYPE == TRA_INT2 && MATRIX) {
+    // The four 2-bit fields of every byte, two field positions per pair of
+    // matrix instructions; element 4 * k + e is field e of byte k.
+#pragma unroll
+    for (int e = 0; e < 4; e += 2) {
+      const uint32_t m0 = (x >> (2 * e)) & 0x03030303u;
+      const uint32_t m1 = (x >> (2 * e + 2)) & 0x03030303u;
+      const long data = (long)(((unsigned long long)m1 << 32) | m0);
+      const float4_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+      const float4_t l = __builtin_amdgcn_mfma_f32_16x16x32_bf8_fp8(sel0, data, z, 0, 0, 0);
+      const float4_t h = __builtin_amdgcn_mfma_f32_16x16x32_bf8_fp8(sel1, data, z, 0, 0, 0);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        fma_step(acc[4 * k + e], s, l[k], b);
+        fma_step(acc[4 * k + e + 1], s, h[k], b);
+      }
+    }
   } else if constexpr (DTYPE == TRA_INT2 && !WEIGHTED) {
     // Same FP8 reading as for int4, on the four 2-bit fields of every byte.
     const float s9 = s * 512.0f;
@@ -225,16 +277,13 @@ __device__ __forceinline__ void accumulate_dword(float* acc, uint32_t x, float s
       fma_step(acc[12 + e], s9, m23.y, b);
     }
   } else if constexpr (DTYPE == TRA_INT2) {
-    float se = s;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const uint32_t m =
-          WEIGHTED ? ((x >> (2 * e)) & 0x03030303u) : (x & (0x03030303u << (2 * e)));
-      fma_step(acc[0 + e], se, byte_to_float<0>(m), b);
-      fma_step(acc[4 + e], se, byte_to_float<1>(m), b);
-      fma_step(acc[8 + e], se, byte_to_float<2>(m), b);
-      fma_step(acc[12 + e], se, byte_to_float<3>(m), b);
-      if constexpr (!WEIGHTED) se *= 0.25f;
+      const uint32_t m = (x >> (2 * e)) & 0x03030303u;
+      fma_step(acc[0 + e], s, byte_to_float<0>(m), b);
+      fma_step(acc[4 + e], s, byte_to_float<1>(m), b);
+      fma_step(acc[8 + e], s, byte_to_float<2>(m), b);
+      fma_step(acc[12 + e], s, byte_to_float<3>(m), b);
     }
   } else if constexpr (DTYPE == TRA_FP16) {
     // s carries the per-sample weight (1.0f when unweighted).
@@ -270,6 +319,9 @@ struct RowWalk {
   // Where a lane loads the dword in front of its chunk together with the chunk
   // (header_with_chunk), the row's header arrives in the row's first lane.
   int hdr_lane;
+  // Selector operands of the matrix instruction that converts int4 / int2
+  // fields (mfma_byte_selector); they depend on the lane only.
+  long sel0, sel1;
   // position weighting: this bag's weight vector (always readable), its last
   // index, whether the feature has one at all, and where the bag starts
   const float* pw;
@@ -384,7 +436,11 @@ __device__ __forceinline__ int fetch_row(RowBuf<CB>& r, IdxT id, IdxT j, IdxT la
 // starts at +0 and a round-to-nearest sum is -0 only if both addends are), and
 // q is a finite integer.  For fp16 / fp32 rows the payload of an invalid row is
 // zeroed as well, so a stored inf / nan in row 0 cannot leak in.
-template <int DTYPE, int CB, bool WEIGHTED>
+// WHOLE_WAVE: every lane of the wave is executing (the pooling loops: their
+// trip counts are wave-uniform and skipped rows are masked, never branched
+// around).  The matrix instruction reads its operands from all 64 lanes
+// whatever the execution mask, so it is used only there.
+template <int DTYPE, int CB, bool WEIGHTED, bool WHOLE_WAVE = true>
 __device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r0, const RowWalk& w) {
   constexpr int EPD = 32 / Traits<DTYPE>::kBits;  // elements per dword
   RowBuf<CB> r = r0;
@@ -404,14 +460,20 @@ __device__ __forceinline__ void consume_row(float* acc, const RowBuf<CB>& r0, co
       s = half_bits_to_float(hdr & 0xffffu);
       b = half_bits_to_float(hdr >> 16);
     }
+    // int4 fields go through the matrix core where a lane holds at most 16
+    // accumulators (8-byte chunks), int2 fields always.
+    constexpr bool kMatrix =
+        WHOLE_WAVE && (Traits<DTYPE>::kBits == 2 || (Traits<DTYPE>::kBits == 4 && CB <= 8));
+    if constexpr (kMatrix)
+      asm volatile("" : "+v"(s));  // the converted scale stays in a register: no fp16 operand in the fused multiply-adds
 #pragma unroll
     for (int i = 0; i < CB / 4; ++i)
-      accumulate_dword<DTYPE, WEIGHTED>(acc + i * EPD, r.d.v[i], s, b);
+      accumulate_dword<DTYPE, WEIGHTED, kMatrix>(acc + i * EPD, r.d.v[i], s, b, w.sel0, w.sel1);
   } else {
     s = r.valid ? r.w : 0.0f;
 #pragma unroll
     for (int i = 0; i < CB / 4; ++i)
-      accumulate_dword<DTYPE, WEIGHTED>(acc + i * EPD, r.valid ? r.d.v[i] : 0u, s, 0.0f);
+      accumulate_dword<DTYPE, WEIGHTED, false>(acc + i * EPD, r.valid ? r.d.v[i] : 0u, s, 0.0f, 0, 0);
   }
 }
 
@@ -1068,6 +1130,8 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_pooled_kernel(const LookupA
   w.set_rows(d.rows, d.row_bytes);
   w.count_errors = c == 0 && d.payload_off == 0;
   w.hdr_lane = lane - c;
+  w.sel0 = mfma_byte_selector(lane, 0);
+  w.sel1 = mfma_byte_selector(lane, 1);
   w.set_position_weights(a, ci, start);
 
   float acc[NE];
@@ -1421,6 +1485,10 @@ __global__ __launch_bounds__(kCuThreads) void tbe_pooled_cu_kernel(
     w.set_rows(d.rows, d.row_bytes);
     w.count_errors = c == 0 && d.payload_off == 0;
     w.hdr_lane = lane - c;
+    w.sel0 = mfma_byte_selector(lane, 0);
+    w.sel1 = mfma_byte_selector(lane, 1);
+  w.sel0 = mfma_byte_selector(lane, 0);
+  w.sel1 = mfma_byte_selector(lane, 1);
     w.set_position_weights(a, sc.first + fi, start);
 
     float acc[NE];
@@ -1477,6 +1545,8 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
   w.set_rows(d.rows, d.row_bytes);
   w.count_errors = c == 0 && d.payload_off == 0;
   w.hdr_lane = lane - c;
+  w.sel0 = mfma_byte_selector(lane, 0);
+  w.sel1 = mfma_byte_selector(lane, 1);
   for (int64_t j = first + (int64_t)tile * rows_per_block + wave * gpw + g; j < last;
        j += stride) {
     RowBuf<CB> r;
@@ -1487,7 +1557,7 @@ __global__ __launch_bounds__(kBlockThreads) void tbe_nobag_kernel(const LookupAr
     float acc[NE];
 #pragma unroll
     for (int i = 0; i < NE; ++i) acc[i] = 0.0f;
-    consume_row<DTYPE, CB, false>(acc, r, w);
+    consume_row<DTYPE, CB, false, /*WHOLE_WAVE=*/false>(acc, r, w);  // lanes leave this loop one by one
     store_outputs<NE>(a, j * (int64_t)d.dim + d.payload_off * 8 / Traits<DTYPE>::kBits + (int64_t)c * NE,
                       acc);
   }
